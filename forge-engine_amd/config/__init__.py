@@ -2,9 +2,10 @@
 
 from .engine import EngineConfig, SchedulerConfig
 from .model import ConfigError, ModelConfig, load_model_config
+from .malusun import MalusunConfig
 from .mazanex import MazanexConfig
 from .qwen3 import Qwen3Config
 from .rekezen import RekezenConfig
 
-__all__ = ["ConfigError", "EngineConfig", "MazanexConfig", "ModelConfig", "Qwen3Config", "RekezenConfig", "SchedulerConfig",
+__all__ = ["ConfigError", "EngineConfig", "MalusunConfig", "MazanexConfig", "ModelConfig", "Qwen3Config", "RekezenConfig", "SchedulerConfig",
            "load_model_config"]

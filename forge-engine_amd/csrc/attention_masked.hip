@@ -6,7 +6,8 @@
 //     (the running maximum starts at sink_h and the running sum at 1);
 //   * values of another width than keys;
 //   * an output gate: the result times sigmoid(gate), a gate per element or one per query head;
-//   * a soft cap: scores, after the scale, become cap * tanh(score / cap).
+//   * a soft cap: scores, after the scale, become cap * tanh(score / cap);
+//   * a penalty on distance: slope_h * (p - j) comes off head h's score of key j (after scale and cap).
 // One launch serves portions of prompts and single tokens alike; the step's own keys and values are
 // already in the pages (keys [page][kv head][slot][D], values transposed [page][kv head][Dv][slot]).
 // Block = (tile of 16 rows, kv head, sequence), a row being a (query token, head of the group) pair,
@@ -23,7 +24,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     T* __restrict__ out, const T* __restrict__ gate, size_t gate_stride, const float* __restrict__ sink,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int D, int Dv, int block_size, int num_blocks, int window,
-    int chunk, float scale, float softcap, int head_gate) {
+    int chunk, float scale, float softcap, int head_gate, const float* __restrict__ slopes) {
   constexpr int KPT = TK / 16;
   extern __shared__ float smem[];
   const int ks = D + 1, vs = Dv + 1;
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
   }
 
   const int head = hk * groups + my_g;
+  const float slope = slopes ? slopes[head] : 0.f;
   float m = sink ? sink[head] : -INFINITY;
   float l = sink ? 1.f : 0.f;
   float acc[DPT];
@@ -120,6 +122,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
       const bool visible = row_ok && kp <= my_pos && kp >= my_first;
       float score = s[i] * scale;
       if (softcap > 0.f) score = softcap * tanhf(score / softcap);
+      if (slopes) score -= slope * (float)(my_pos - kp);
       s[i] = visible ? score : -INFINITY;
       tile_max = fmaxf(tile_max, s[i]);
     }
@@ -180,7 +183,7 @@ static int launch_masked(const void* q, long long q_stride, const void* key_page
                          const void* gate, long long gate_stride, const float* sink, const int* cu_q,
                          const int* ctx_len, const int* block_table, int table_stride, int num_seqs, int max_q_len,
                          int q_heads, int kv_heads, int D, int Dv, int block_size, int num_blocks, int window,
-                         int chunk, float scale, float softcap, int head_gate, hipStream_t stream) {
+                         int chunk, float scale, float softcap, int head_gate, const float* slopes, hipStream_t stream) {
   const int groups = q_heads / kv_heads;
   const long long rows = (long long)max_q_len * groups;
   const dim3 grid((unsigned)((rows + ROWS - 1) / ROWS), kv_heads, num_seqs);
@@ -190,7 +193,7 @@ static int launch_masked(const void* q, long long q_stride, const void* key_page
   masked_attention_kernel<T, TK, DPT><<<grid, 256, lds, stream>>>(                                               \
       (const T*)q, (size_t)q_stride, (const T*)key_pages, (const T*)value_pages, (T*)out, (const T*)gate,        \
       (size_t)gate_stride, sink, cu_q, ctx_len, block_table, table_stride, kv_heads, groups, D, Dv, block_size, \
-      num_blocks, window, chunk, scale, softcap, head_gate)
+      num_blocks, window, chunk, scale, softcap, head_gate, slopes)
   if (tk == 32) {
     if (Dv <= 64) LAUNCH(32, 4);
     else if (Dv <= 128) LAUNCH(32, 8);
@@ -209,7 +212,8 @@ extern "C" int fe_masked_attention(const void* q, int dtype, long long q_stride,
                                    const float* sink, const int* cu_q, const int* ctx_len, const int* block_table,
                                    int table_stride, int num_seqs, int max_q_len, int q_heads, int kv_heads,
                                    int head_dim, int value_dim, int block_size, int num_blocks, int window, int chunk,
-                                   float scale, float softcap, int head_gate, int tokens, hipStream_t stream) {
+                                   float scale, float softcap, int head_gate, int tokens, const float* slopes,
+                                   hipStream_t stream) {
   if (tokens <= 0 || num_seqs <= 0) return FE_OK;
   if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || head_dim < 1 || head_dim > 256 || value_dim < 1 ||
       value_dim > 256 || block_size <= 0 || num_blocks <= 0 || max_q_len < 1 || window < 0 || chunk < 0 ||
@@ -221,10 +225,10 @@ extern "C" int fe_masked_attention(const void* q, int dtype, long long q_stride,
   if (dtype == FE_F32)
     return launch_masked<float>(q, q_stride, key_pages, value_pages, out, gate, gate_stride, sink, cu_q, ctx_len,
                                 block_table, table_stride, num_seqs, max_q_len, q_heads, kv_heads, head_dim, value_dim,
-                                block_size, num_blocks, window, chunk, scale, softcap, head_gate, stream);
+                                block_size, num_blocks, window, chunk, scale, softcap, head_gate, slopes, stream);
   if (dtype == FE_BF16)
     return launch_masked<bf16_t>(q, q_stride, key_pages, value_pages, out, gate, gate_stride, sink, cu_q, ctx_len,
                                  block_table, table_stride, num_seqs, max_q_len, q_heads, kv_heads, head_dim, value_dim,
-                                 block_size, num_blocks, window, chunk, scale, softcap, head_gate, stream);
+                                 block_size, num_blocks, window, chunk, scale, softcap, head_gate, slopes, stream);
   return FE_BAD_ARGUMENT;
 }

@@ -9,6 +9,9 @@
 // The projection's bias (float32, one entry per q, k and v channel, or none) is added here, to the
 // rows as they are loaded, so that the product before this kernel has none; the state holds rows
 // with their bias.  One wave per token and head; everything between the loads and the stores is float32.
+// Values may lean on another layer's values of the same tokens: v <- (1 - mix) v + mix * v_from
+// (v_from [T, kv_heads * value_dim], dense), after the bias and the convolution and before the page
+// write; a layer that others lean on leaves its values, as stored, in v_keep (same shape).
 #include "common.h"
 
 #define CR_THREADS 256
@@ -23,7 +26,7 @@ __global__ __launch_bounds__(64) void conv_rope_norm_write_kernel(
     const int* __restrict__ state_slots, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ key_pages, T* __restrict__ value_pages, T* __restrict__ q_out, int q_heads, int kv_heads,
     int head_dim, int value_dim, int rotary_dim, float eps, int unit_norm, int taps, int block_size,
-    int num_blocks, int slots) {
+    int num_blocks, int slots, const T* __restrict__ v_from, float v_mix, T* __restrict__ v_keep) {
   __shared__ float y[CR_HEAD_MAX];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int seq = token_seq[t];
@@ -62,10 +65,13 @@ __global__ __launch_bounds__(64) void conv_rope_norm_write_kernel(
   const int place = pos % block_size;
   const bool paged = page >= 0 && page < num_blocks;
   if (is_v) {
-    if (paged) {
-      const int hv = head - q_heads - kv_heads;
-      for (int d = lane; d < n; d += 64)
-        store_from_float(value_pages + (((size_t)page * kv_heads + hv) * value_dim + d) * block_size + place, y[d]);
+    const int hv = head - q_heads - kv_heads;
+    const size_t dense = (size_t)t * v_size + (size_t)hv * value_dim;
+    for (int d = lane; d < n; d += 64) {
+      float v = y[d];
+      if (v_from) v = (1.f - v_mix) * v + v_mix * load_as_float(v_from + dense + d);
+      if (v_keep) store_from_float(v_keep + dense + d, v);
+      if (paged) store_from_float(value_pages + (((size_t)page * kv_heads + hv) * value_dim + d) * block_size + place, v);
     }
     return;
   }
@@ -130,7 +136,8 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
                                        const int* block_table, int table_stride, void* key_pages, void* value_pages,
                                        void* q_out, int tokens, int q_heads, int kv_heads, int head_dim, int value_dim,
                                        int rotary_dim, float eps, int unit_norm, int taps, int block_size,
-                                       int num_blocks, int slots, hipStream_t stream) {
+                                       int num_blocks, int slots, const void* v_from, float v_mix, void* v_keep,
+                                       hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
   if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || value_dim <= 0 || block_size <= 0 || num_blocks <= 0)
     return FE_BAD_ARGUMENT;
@@ -145,7 +152,7 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
   conv_rope_norm_write_kernel<T><<<grid, 64, 0, stream>>>(                                         \
       (const T*)qkv, (size_t)qkv_stride, bias, conv_w, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, \
       block_table, table_stride, (T*)key_pages, (T*)value_pages, (T*)q_out, q_heads, kv_heads, head_dim,       \
-      value_dim, rotary_dim, eps, unit_norm, taps, block_size, num_blocks, slots)
+      value_dim, rotary_dim, eps, unit_norm, taps, block_size, num_blocks, slots, (const T*)v_from, v_mix, (T*)v_keep)
   if (dtype == FE_F32) LAUNCH(float);
   else if (dtype == FE_BF16) LAUNCH(bf16_t);
   else return FE_BAD_ARGUMENT;

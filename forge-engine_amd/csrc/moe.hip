@@ -2,9 +2,11 @@
 // two grouped matrix products over the sorted rows.  Nothing is decided on the host.
 //
 //   fe_moe_select:   from router logits (float32): bias added, the `top` largest per token, softmax over those alone
+//                    (or, scoring 1, each chosen logit's own sigmoid)
 //   fe_moe_plan:     counts per expert, their prefix sums, and the pairs ordered by expert
 //   fe_moe_gate_up:  for every pair, act = min(g, L) * sigmoid(alpha min(g, L)) * (clamp(u, -L, L) + 1) with
-//                    g = W_gate[e] x, u = W_up[e] x of the pair's token and expert
+//                    g = W_gate[e] x, u = W_up[e] x of the pair's token and expert (form 1: silu(g) * u; with
+//                    input weights, g and u are first multiplied by the pair's routing weight)
 //   fe_moe_down:     out[choice][token] = weight * W_down[e] act   (float32; one part per choice, so
 //                    that the reader adds a token's experts up in a fixed order; the first choice's part
 //                    also takes what every token gets beside its experts, a shared expert's output)
@@ -22,12 +24,12 @@
 // caller): bias added, the `top` largest chosen one after the other (the largest first; among equals
 // the lowest index), weights = softmax over the chosen logits alone.
 __global__ void moe_select_kernel(const float* __restrict__ z, const float* __restrict__ bias, int* __restrict__ chosen,
-                                  float* __restrict__ weights, int tokens, int E, int top) {
+                                  float* __restrict__ weights, int tokens, int E, int top, int scoring) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= tokens) return;
   const float* row = z + (size_t)t * E;
   int picked[16];
-  float best[16];
+  float best[16], raw[16];
   float peak = 0.f, denom = 0.f;
   for (int k = 0; k < top; ++k) {
     int arg = -1;
@@ -44,17 +46,20 @@ __global__ void moe_select_kernel(const float* __restrict__ z, const float* __re
     picked[k] = arg;
     chosen[(size_t)t * top + k] = arg;
     if (k == 0) peak = value;
+    raw[k] = value;
     best[k] = expf(value - peak);
     denom += best[k];
   }
-  for (int k = 0; k < top; ++k) weights[(size_t)t * top + k] = best[k] / denom;
+  // scoring 1: a chosen expert's weight is the sigmoid of its own logit, whatever the others are
+  for (int k = 0; k < top; ++k)
+    weights[(size_t)t * top + k] = scoring == 1 ? 1.f / (1.f + expf(-raw[k])) : best[k] / denom;
 }
 
 extern "C" int fe_moe_select(const float* logits, const float* bias, int* chosen, float* weights, int tokens, int experts,
-                             int top, hipStream_t stream) {
+                             int top, int scoring, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
-  if (experts <= 0 || experts > 1024 || top < 1 || top > 16 || top > experts) return FE_BAD_ARGUMENT;
-  moe_select_kernel<<<(tokens + 63) / 64, 64, 0, stream>>>(logits, bias, chosen, weights, tokens, experts, top);
+  if (experts <= 0 || experts > 1024 || top < 1 || top > 16 || top > experts || scoring < 0 || scoring > 1) return FE_BAD_ARGUMENT;
+  moe_select_kernel<<<(tokens + 63) / 64, 64, 0, stream>>>(logits, bias, chosen, weights, tokens, experts, top, scoring);
   return fe_check_launch();
 }
 
@@ -97,7 +102,12 @@ extern "C" int fe_moe_plan(const int* chosen, int pairs, int experts, int* offse
 #define BN 64
 #define BK 32
 
-__device__ __forceinline__ float gated(float g, float u, float limit, float alpha) {
+// form 0: the bounded activation above; form 1: silu(g) * u.  `w` scales both products first (a router's weight
+// on the expert's input: W (w x) = w (W x)).
+__device__ __forceinline__ float gated(float g, float u, float limit, float alpha, int form, float w) {
+  g *= w;
+  u *= w;
+  if (form == 1) return g / (1.f + expf(-g)) * u;
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);
@@ -139,7 +149,7 @@ template <typename T, int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const T* __restrict__ a, const T* __restrict__ w, const int* __restrict__ offsets, const int* __restrict__ order,
     const float* __restrict__ pair_weight, T* __restrict__ act, float* __restrict__ out, int E, int N, int K, int top,
-    int tokens, float limit, float alpha, const float* __restrict__ extra, int extra_parts) {
+    int tokens, float limit, float alpha, int form, const float* __restrict__ extra, int extra_parts) {
   __shared__ float As[BM][BK + 1];
   __shared__ float Ws[BN][BK + 1];
   __shared__ float Us[MODE == 0 ? BN : 1][BK + 1];
@@ -205,11 +215,11 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       const int n = n0 + tx + 16 * j;
       if (n >= N) continue;
       if (MODE == 0) {
-        store_from_float(act + (size_t)(row0 + r) * N + n, gated(acc_g[i][j], acc_u[i][j], limit, alpha));
+        store_from_float(act + (size_t)(row0 + r) * N + n, gated(acc_g[i][j], acc_u[i][j], limit, alpha, form, pair_weight ? pair_weight[pair] : 1.f));
       } else {
         const int token = pair / top, choice = pair - token * top;
         out[((size_t)choice * tokens + token) * N + n] =
-            with_extra(acc_g[i][j] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
+            with_extra(acc_g[i][j] * (pair_weight ? pair_weight[pair] : 1.f), choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
       }
     }
   }
@@ -243,7 +253,7 @@ template <int MODE, int NT, int MT>
 __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
     const int* __restrict__ order, const float* __restrict__ pair_weight, bf16_t* __restrict__ act,
-    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha,
+    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha, int form,
     const float* __restrict__ extra, int extra_parts, int slots, int column_tiles) {
   // NT: groups of 16 columns a wave (a block takes 64 NT columns); MT: tiles of 16 rows a wave (a block takes
   // 16 MT rows, every wave all of them).  Steps of few rows launch <MODE, 1, 4>: many blocks, each streaming
@@ -364,11 +374,11 @@ __global__ __launch_bounds__(256) void moe_grouped_mfma_kernel(
         const int pair = pair_of[r];
         if (pair < 0) continue;
         if (MODE == 0) {
-          act[(size_t)(row0 + r) * N + n[nt]] = float_to_bf16(gated(acc_g[nt][mt][i], acc_u[nt][mt][i], limit, alpha));
+          act[(size_t)(row0 + r) * N + n[nt]] = float_to_bf16(gated(acc_g[nt][mt][i], acc_u[nt][mt][i], limit, alpha, form, pair_weight ? pair_weight[pair] : 1.f));
         } else {
           const int token = pair / top, choice = pair - token * top;
           out[((size_t)choice * tokens + token) * N + n[nt]] = with_extra(
-              acc_g[nt][mt][i] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n[nt]);
+              acc_g[nt][mt][i] * (pair_weight ? pair_weight[pair] : 1.f), choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n[nt]);
         }
       }
   }
@@ -391,7 +401,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_staged_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ offsets,
     const int* __restrict__ order, const float* __restrict__ pair_weight, bf16_t* __restrict__ act,
-    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha,
+    float* __restrict__ out, int E, int N, int K, int top, int tokens, float limit, float alpha, int form,
     const float* __restrict__ extra, int extra_parts, int slots, int column_tiles) {
   constexpr int COLS = 128, MATS = MODE == 0 ? 2 : 1, NT = 2, MT = 4;
   __shared__ __attribute__((aligned(16))) bf16_t As[2][TM][TPAD];
@@ -498,11 +508,11 @@ __global__ __launch_bounds__(256) void moe_grouped_staged_kernel(
         const int pair = pair_of[r];
         if (pair < 0) continue;
         if (MODE == 0) {
-          act[(size_t)(row0 + r) * N + n] = float_to_bf16(gated(acc[0][nt][mt][i], acc[MATS - 1][nt][mt][i], limit, alpha));
+          act[(size_t)(row0 + r) * N + n] = float_to_bf16(gated(acc[0][nt][mt][i], acc[MATS - 1][nt][mt][i], limit, alpha, form, pair_weight ? pair_weight[pair] : 1.f));
         } else {
           const int token = pair / top, choice = pair - token * top;
           out[((size_t)choice * tokens + token) * N + n] = with_extra(
-              acc[0][nt][mt][i] * pair_weight[pair], choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
+              acc[0][nt][mt][i] * (pair_weight ? pair_weight[pair] : 1.f), choice, extra, extra_parts, (size_t)tokens * N, (size_t)token * N + n);
         }
       }
   }
@@ -518,17 +528,17 @@ static unsigned mfma_blocks(int slots, int column_tiles) { return (unsigned)(((l
 // (a prompt of 2,048 tokens at a width of 2,048: 3.80 -> 3.67 ms against the direct shape with two column groups
 // a wave; at 4,096: 10.0 -> 9.6 ms, where the direct shape with blocks of 128 rows reached 9.9), below that the
 // direct shape with one column group a wave, which streams the weight at 3 to 4.7 TB/s in a decode step.
-#define MFMA_LAUNCH(MODE, COLUMNS, A, W, PW, ACT, OUT, N_, K_, LIMIT, ALPHA, EXTRA, EXTRA_PARTS)                          \
+#define MFMA_LAUNCH(MODE, COLUMNS, A, W, PW, ACT, OUT, N_, K_, LIMIT, ALPHA, FORM, EXTRA, EXTRA_PARTS)                        \
   do {                                                                                                                   \
     const bool wide = pairs >= WIDE_COLUMNS_MIN_PAIRS;                                                                   \
     const int slots = (int)(pairs / TM + experts);                                                                       \
     const int tiles = ((COLUMNS) + (wide ? 2 : 1) * TN - 1) / ((wide ? 2 : 1) * TN);                                      \
     if (wide)                                                                                                            \
       moe_grouped_staged_kernel<MODE><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                    \
-          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
+          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, FORM, EXTRA, EXTRA_PARTS, slots, tiles); \
     else                                                                                                                 \
       moe_grouped_mfma_kernel<MODE, 1, 4><<<mfma_blocks(slots, tiles), 256, 0, stream>>>(                                \
-          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, EXTRA, EXTRA_PARTS, slots, tiles); \
+          A, W, offsets, order, PW, ACT, OUT, experts, N_, K_, top, tokens, LIMIT, ALPHA, FORM, EXTRA, EXTRA_PARTS, slots, tiles); \
   } while (0)
 
 static bool mfma_fits(const void* a, const void* w, int K) {
@@ -536,21 +546,23 @@ static bool mfma_fits(const void* a, const void* w, int K) {
 }
 
 extern "C" int fe_moe_gate_up(const void* x, const void* gate_up, int dtype, const int* offsets, const int* order, void* act,
-                              int tokens, int top, int experts, int hidden, int inner, float limit, float alpha,
-                              hipStream_t stream) {
+                              int tokens, int top, int experts, int hidden, int inner, float limit, float alpha, int form,
+                              const float* input_weight, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
-  if (top < 1 || experts < 1 || experts > 1024 || hidden <= 0 || inner <= 0 || !(limit > 0.f)) return FE_BAD_ARGUMENT;
+  if (top < 1 || experts < 1 || experts > 1024 || hidden <= 0 || inner <= 0 || form < 0 || form > 1 ||
+      (form == 0 && !(limit > 0.f)))
+    return FE_BAD_ARGUMENT;
   const long long pairs = (long long)tokens * top;
   const dim3 grid((unsigned)(pairs / BM + experts), (unsigned)((inner + BN - 1) / BN));
   if (dtype == FE_F32)
-    moe_grouped_kernel<float, 0><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, offsets, order, nullptr,
-                                                           (float*)act, nullptr, experts, inner, hidden, top, tokens, limit, alpha, nullptr, 0);
+    moe_grouped_kernel<float, 0><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, offsets, order, input_weight,
+                                                           (float*)act, nullptr, experts, inner, hidden, top, tokens, limit, alpha, form, nullptr, 0);
   else if (dtype == FE_BF16 && mfma_fits(x, gate_up, hidden)) {
-    MFMA_LAUNCH(0, inner, (const bf16_t*)x, (const bf16_t*)gate_up, nullptr, (bf16_t*)act, nullptr, inner, hidden, limit, alpha, nullptr, 0);
+    MFMA_LAUNCH(0, inner, (const bf16_t*)x, (const bf16_t*)gate_up, input_weight, (bf16_t*)act, nullptr, inner, hidden, limit, alpha, form, nullptr, 0);
   } else if (dtype == FE_BF16)
-    moe_grouped_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, nullptr,
+    moe_grouped_kernel<bf16_t, 0><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, offsets, order, input_weight,
                                                             (bf16_t*)act, nullptr, experts, inner, hidden, top, tokens, limit,
-                                                            alpha, nullptr, 0);
+                                                            alpha, form, nullptr, 0);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();
@@ -565,13 +577,13 @@ extern "C" int fe_moe_down(const void* act, const void* down, int dtype, const i
   const dim3 grid((unsigned)(pairs / BM + experts), (unsigned)((hidden + BN - 1) / BN));
   if (dtype == FE_F32)
     moe_grouped_kernel<float, 1><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, offsets, order, pair_weight,
-                                                           nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, extra,
+                                                           nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, 0, extra,
                                                            extra_parts);
   else if (dtype == FE_BF16 && mfma_fits(act, down, inner)) {
-    MFMA_LAUNCH(1, hidden, (const bf16_t*)act, (const bf16_t*)down, pair_weight, nullptr, out, hidden, inner, 0.f, 0.f, extra, extra_parts);
+    MFMA_LAUNCH(1, hidden, (const bf16_t*)act, (const bf16_t*)down, pair_weight, nullptr, out, hidden, inner, 0.f, 0.f, 0, extra, extra_parts);
   } else if (dtype == FE_BF16)
     moe_grouped_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, offsets, order, pair_weight,
-                                                            nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, extra,
+                                                            nullptr, out, experts, hidden, inner, top, tokens, 0.f, 0.f, 0, extra,
                                                            extra_parts);
   else
     return FE_BAD_ARGUMENT;
@@ -587,7 +599,7 @@ __global__ void gated_act_kernel(const T* __restrict__ gate_up, T* __restrict__ 
   const long long t = i / inner;
   const int n = (int)(i - t * inner);
   const T* row = gate_up + t * 2 * inner;
-  store_from_float(out + i, gated(load_as_float(row + n), load_as_float(row + inner + n), limit, alpha));
+  store_from_float(out + i, gated(load_as_float(row + n), load_as_float(row + inner + n), limit, alpha, 0, 1.f));
 }
 
 extern "C" int fe_gated_act(const void* gate_up, void* out, int dtype, int tokens, int inner, float limit, float alpha,

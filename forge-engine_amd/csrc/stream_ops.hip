@@ -285,6 +285,25 @@ extern "C" int fe_tanh_rows(void* x, int dtype, long long count, hipStream_t str
   return fe_check_launch();
 }
 
+// The square of relu over every element, float32 inside.
+template <typename T>
+__global__ void relu_squared_kernel(const T* __restrict__ x, T* __restrict__ out, long long count) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const float v = fmaxf(load_as_float(x + i), 0.f);
+  store_from_float(out + i, v * v);
+}
+
+extern "C" int fe_relu_squared(const void* x, void* out, int dtype, long long count, hipStream_t stream) {
+  if (count <= 0) return FE_OK;
+  const long long blocks = (count + 255) / 256;
+  if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  if (dtype == FE_F32) relu_squared_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)x, (float*)out, count);
+  else if (dtype == FE_BF16) relu_squared_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, count);
+  else return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
 // ---------------------------------------------------------------- per-head norm, weight and gate
 // One wave per (token, head): y = o[:dim] (divided by max(|o[dim]|, floor) + 1e-6 with a normaliser
 // column), y / rms(y) * weight * act(gate).

@@ -46,6 +46,9 @@ class StepBatch:
     q_lens: list
     ctx_before_host: list
     state_slots_host: list
+    # what a layer of the step leaves for later layers of the same step, by name (device tensors over the
+    # step's tokens: the values that later layers' values lean on)
+    carry: dict = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

@@ -1177,7 +1177,7 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
                          positions: Tensor, token_seq: Tensor, cu_q: Tensor, state_slots: Tensor, block_table: Tensor,
                          key_pages: Tensor, value_pages: Tensor, q_out: Tensor, *, num_seqs: int, q_heads: int,
                          kv_heads: int, head_dim: int, value_dim: int, rotary_dim: int, unit_norm_eps: float | None,
-                         taps: int) -> None:
+                         taps: int, v_from: Tensor | None = None, v_mix: float = 0.0, v_keep: Tensor | None = None) -> None:
     """From the projection's output to queries and cached keys and values in one kernel: a short
     projection's bias (float32 [channels] or None: the product before has none), a short causal
     convolution over time on every q, k and v channel (``taps`` > 0: y_t = sum_j c[:, j] *
@@ -1186,7 +1186,9 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
     ``rotary_dim`` dims of q and k heads (dim i pairs with i + rotary_dim / 2); then q and k heads
     divided by their root mean square (``unit_norm_eps`` not None); q into ``q_out`` [T, Hq * D],
     k and v into their pages (values transposed).  float32 inside, one rounding at the stores.
-    qkv [T, >= channels] with any row stride."""
+    qkv [T, >= channels] with any row stride.  ``v_from`` ([T, kv_heads * value_dim], another layer's values of
+    the same tokens): the values become ``(1 - v_mix) v + v_mix v_from`` before they are stored; ``v_keep`` (same
+    shape) receives the values as stored, for layers that lean on this one's."""
     channels = (q_heads + kv_heads) * head_dim + kv_heads * value_dim
     _gpu(qkv, "qkv", contiguous=False)
     tokens = qkv.shape[0]
@@ -1228,6 +1230,11 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
         raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {value_dim}, block_size], got {tuple(value_pages.shape)}")
     if block_table.dim() != 2 or block_table.stride(1) != 1 or block_table.shape[0] < num_seqs:
         raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
+    for name, dense in (("v_from", v_from), ("v_keep", v_keep)):
+        if dense is not None:
+            _gpu(dense, name, qkv.dtype)
+            if dense.shape != (tokens, kv_heads * value_dim):
+                raise KernelError(f"{name} must be [{tokens}, {kv_heads * value_dim}], got {tuple(dense.shape)}")
     stride = qkv.stride(0) if tokens > 1 else max(qkv.stride(0), qkv.shape[1])
     slots = conv_state.shape[0] if taps > 1 else 0
     _call("conv_rope", "fe_conv_rope_norm_write", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(bias),
@@ -1236,7 +1243,7 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
           _ptr(key_pages), _ptr(value_pages), _ptr(q_out), c_int(tokens), c_int(q_heads), c_int(kv_heads), c_int(head_dim),
           c_int(value_dim), c_int(rotary_dim), c_float(unit_norm_eps if unit_norm_eps is not None else 0.0),
           c_int(1 if unit_norm_eps is not None else 0), c_int(taps), c_int(block_size), c_int(num_blocks), c_int(slots),
-          _stream())
+          _ptr(v_from), c_float(v_mix), _ptr(v_keep), _stream())
     if taps > 1:
         _call("conv_rope", "fe_conv_state_update", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(bias), _ptr(conv_state),
               _ptr(cu_q), _ptr(state_slots), c_int(num_seqs), c_int(channels), c_int(taps), c_int(slots), c_int(tokens),
@@ -1247,13 +1254,15 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
                      block_table: Tensor, *, num_seqs: int, max_q_len: int, q_heads: int, kv_heads: int, head_dim: int,
                      value_dim: int, scale: float, window: int | None = None, chunk: int | None = None,
                      sink: Tensor | None = None, gate: Tensor | None = None, num_decode: int | None = None,
-                     max_ctx: int | None = None, softcap: float | None = None, head_gate: bool = False) -> Tensor:
+                     max_ctx: int | None = None, softcap: float | None = None, head_gate: bool = False,
+                     slopes: Tensor | None = None) -> Tensor:
     """Paged grouped-query attention with the masks and softmax forms beyond the causal one: the
     query at position p reads keys j <= p with j > p - window (``window``) and j >= p - p % chunk
     (``chunk``); ``sink`` (float32 [Hq]) adds exp(sink_h) to head h's softmax denominator, with
     no key and no value; values may be of another width than keys; ``gate`` ([T, Hq * Dv] rows of
     any stride; with ``head_gate`` [T, Hq], one number a head) multiplies the result by sigmoid(gate);
-    ``softcap``: scores, after the scale, become cap * tanh(score / cap).  out [T, Hq * Dv].  Scores and softmax
+    ``softcap``: scores, after the scale, become cap * tanh(score / cap); ``slopes`` (float32 [Hq]): head h's score
+    of key j loses slopes[h] * (p - j).  out [T, Hq * Dv].  Scores and softmax
     float32.  A bfloat16 cache with keys and values of 64 or 128 elements, groups up to 8 and pages of
     a power of two >= 16 goes to the matrix-core kernels of ``paged_attention`` (single tokens and
     portions each to its own), with the gate in a small kernel behind them; everything else, and
@@ -1284,6 +1293,10 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
         _gpu(sink, "sink", torch.float32)
         if sink.shape != (q_heads,):
             raise KernelError(f"sink must be [{q_heads}]")
+    if slopes is not None:
+        _gpu(slopes, "slopes", torch.float32)
+        if slopes.shape != (q_heads,):
+            raise KernelError(f"slopes must be [{q_heads}]")
     gate_stride = 0
     if gate is not None:
         gate_stride = _strided_rows(gate, "gate", q_heads if head_gate else q_heads * value_dim)
@@ -1293,7 +1306,7 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
         raise KernelError("softcap must be positive")
     if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
         raise KernelError("window, chunk and max_q_len must be positive")
-    if (q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
+    if (slopes is None and q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
             and block_size >= 16 and block_size & (block_size - 1) == 0 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0):
         paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
                         q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window,
@@ -1307,7 +1320,7 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
           _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(q_heads),
           c_int(kv_heads), c_int(head_dim), c_int(value_dim), c_int(block_size), c_int(num_blocks),
           c_int(window or 0), c_int(chunk or 0), c_float(scale), c_float(softcap or 0.0), c_int(1 if head_gate else 0),
-          c_int(tokens), _stream())
+          c_int(tokens), _ptr(slopes), _stream())
     return out
 
 
@@ -1536,10 +1549,14 @@ def whole_norm_rope_write(qkv: Tensor, q_weight: Tensor, k_weight: Tensor | None
 
 # ------------------------------------------------- a mixture of experts
 
-def moe_route(x: Tensor, router_weight: Tensor, router_bias: Tensor | None, top: int) -> tuple[Tensor, Tensor]:
+_SCORINGS = {"softmax": 0, "sigmoid": 1}
+_GATED_FORMS = {"bounded": 0, "silu": 1}
+
+
+def moe_route(x: Tensor, router_weight: Tensor, router_bias: Tensor | None, top: int, scoring: str = "softmax") -> tuple[Tensor, Tensor]:
     """Router logits ``x W^T + b`` in float32; for every token the ``top`` experts with the largest logits
-    (int32 [T, top], largest first, the lowest index among equals) and the softmax over their logits alone
-    (float32 [T, top])."""
+    (int32 [T, top], largest first, the lowest index among equals) and their weights (float32 [T, top]): the
+    softmax over the chosen logits alone, or (``scoring`` "sigmoid") each chosen logit's own sigmoid."""
     _gpu(x, "x")
     _gpu(router_weight, "router_weight", x.dtype)
     tokens, hidden = x.shape
@@ -1554,18 +1571,20 @@ def moe_route(x: Tensor, router_weight: Tensor, router_bias: Tensor | None, top:
     chosen = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
     _call("moe", "fe_moe_select", _ptr(logits), _ptr(router_bias), _ptr(chosen), _ptr(weights), c_int(tokens), c_int(experts),
-          c_int(top), _stream())
+          c_int(top), c_int(_SCORINGS[scoring]), _stream())
     return chosen, weights
 
 
-def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, down: Tensor, out: Tensor, *, limit: float,
-                alpha: float, extra: Tensor | None = None) -> Tensor:
+def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, down: Tensor, out: Tensor, *, limit: float = 0.0,
+                alpha: float = 1.0, extra: Tensor | None = None, form: str = "bounded", weight_input: bool = False) -> Tensor:
     """out[k, t] = weights[t, k] * down[e] @ act, e = chosen[t, k], with ``act = min(g, limit) *
     sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1)``, ``g = gate_up[e, :F] @ x[t]``,
     ``u = gate_up[e, F:] @ x[t]``.  x [T, H]; gate_up [E, 2F, H]; down [E, H, F]; out float32 [top, T, H]
     (one part per choice).  ``extra`` (float32 [T, H] or [parts, T, H], added up in order): what every
-    token gets beside its experts; it joins the first choice's part.  The pairs are sorted by expert on the
-    device and two grouped products run over the sorted rows."""
+    token gets beside its experts; it joins the first choice's part.  ``form`` "silu": ``act = silu(g) * u``, no
+    bounds.  ``weight_input``: the routing weight scales the expert's input instead of its output (g and u are
+    multiplied by it before the activation, which is the same as multiplying x).  The pairs are sorted by
+    expert on the device and two grouped products run over the sorted rows."""
     _gpu(x, "x")
     _gpu(chosen, "chosen", torch.int32)
     _gpu(weights, "weights", torch.float32)
@@ -1583,8 +1602,8 @@ def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, dow
         raise KernelError("chosen and weights must be [T, top <= 16] and experts at most 1,024")
     if out.shape != (top, tokens, hidden):
         raise KernelError(f"out must be [{top}, {tokens}, {hidden}], got {tuple(out.shape)}")
-    if not limit > 0.0:
-        raise KernelError("limit must be positive")
+    if form not in _GATED_FORMS or (form == "bounded" and not limit > 0.0):
+        raise KernelError("the bounded activation needs a positive limit; forms: " + ", ".join(_GATED_FORMS))
     extra_parts = 0 if extra is None else _parts_of(extra, tokens, hidden, "extra")
     pairs = tokens * top
     offsets = torch.empty(experts + 1, dtype=torch.int32, device=x.device)
@@ -1593,8 +1612,9 @@ def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, dow
     code = c_int(_code(x.dtype))
     _call("moe", "fe_moe_plan", _ptr(chosen), c_int(pairs), c_int(experts), _ptr(offsets), _ptr(order), _stream())
     _call("moe", "fe_moe_gate_up", _ptr(x), _ptr(gate_up), code, _ptr(offsets), _ptr(order), _ptr(act), c_int(tokens), c_int(top),
-          c_int(experts), c_int(hidden), c_int(inner), c_float(limit), c_float(alpha), _stream())
-    _call("moe", "fe_moe_down", _ptr(act), _ptr(down), code, _ptr(offsets), _ptr(order), _ptr(weights), _ptr(out), c_int(tokens),
+          c_int(experts), c_int(hidden), c_int(inner), c_float(limit), c_float(alpha), c_int(_GATED_FORMS[form]),
+          _ptr(weights if weight_input else None), _stream())
+    _call("moe", "fe_moe_down", _ptr(act), _ptr(down), code, _ptr(offsets), _ptr(order), _ptr(None if weight_input else weights), _ptr(out), c_int(tokens),
           c_int(top), c_int(experts), c_int(hidden), c_int(inner), _ptr(extra), c_int(extra_parts), _stream())
     return out
 
@@ -1609,4 +1629,112 @@ def linear_gated(x: Tensor, gate_up_weight: Tensor, *, limit: float, alpha: floa
     out = torch.empty((tokens, width // 2), dtype=gate_up.dtype, device=gate_up.device)
     _call("moe", "fe_gated_act", _ptr(gate_up), _ptr(out), c_int(_code(gate_up.dtype)), c_int(tokens), c_int(width // 2),
           c_float(limit), c_float(alpha), _stream())
+    return out
+
+
+# ------------------------------------------------- dense activations, short convolutions, selective scans
+
+def relu_squared(x: Tensor) -> Tensor:
+    """max(x, 0)^2 of every element, into a new tensor of x's dtype (float32 inside)."""
+    _gpu(x, "x")
+    out = torch.empty_like(x)
+    _call("stream_ops", "fe_relu_squared", _ptr(x), _ptr(out), c_int(_code(x.dtype)), c_longlong(x.numel()), _stream())
+    return out
+
+
+def causal_conv_act(u: Tensor, weight: Tensor, bias: Tensor | None, state: Tensor | None, token_seq: Tensor, cu_q: Tensor,
+                    state_slots: Tensor, *, num_seqs: int, act: str = "silu") -> Tensor:
+    """A short causal convolution over time on every channel, then the activation: ``y_t = act(b + sum_j
+    w[:, j] * u_(t - taps + 1 + j))``.  u [T, >= channels] with any row stride (its first ``channels`` columns
+    are read); weight float32 [channels, taps], the last column the token's own; bias float32 [channels] or
+    None; state float32 [slots, taps - 1, channels]: every sequence's last taps - 1 rows of u, read for the
+    rows before the step and moved on afterwards (None with one tap).  Returns [T, channels] in u's dtype."""
+    _gpu(u, "u", contiguous=False)
+    _gpu(weight, "weight", torch.float32)
+    if weight.dim() != 2 or not 1 <= weight.shape[1] <= 8:
+        raise KernelError("weight must be [channels, taps in 1..8]")
+    channels, taps = weight.shape
+    tokens = u.shape[0]
+    stride = _strided_rows(u, "u", channels)
+    if bias is not None:
+        _gpu(bias, "bias", torch.float32)
+        if bias.shape != (channels,):
+            raise KernelError(f"bias must be [{channels}]")
+    if taps > 1:
+        _gpu(state, "state", torch.float32)
+        if state.dim() != 3 or state.shape[1:] != (taps - 1, channels):
+            raise KernelError(f"state must be [slots, {taps - 1}, {channels}]")
+    _gpu(token_seq, "token_seq", torch.int32)
+    if token_seq.numel() != tokens:
+        raise KernelError("token_seq must have one entry per token")
+    _sequences(cu_q, state_slots, num_seqs)
+    if act not in _ACTS or _ACTS[act] > 1:
+        raise KernelError("act must be none or silu")
+    slots = state.shape[0] if taps > 1 else 0
+    out = torch.empty((tokens, channels), dtype=u.dtype, device=u.device)
+    code = c_int(_code(u.dtype))
+    _call("selective_scan", "fe_causal_conv_act", _ptr(u), code, c_longlong(stride), _ptr(weight), _ptr(bias),
+          _ptr(state if taps > 1 else None), _ptr(token_seq), _ptr(cu_q), _ptr(state_slots), _ptr(out), c_int(tokens),
+          c_int(channels), c_int(taps), c_int(slots), c_int(_ACTS[act]), _stream())
+    if taps > 1:
+        _call("conv_rope", "fe_conv_state_update", _ptr(u), code, c_longlong(stride), _ptr(None), _ptr(state), _ptr(cu_q),
+              _ptr(state_slots), c_int(num_seqs), c_int(channels), c_int(taps), c_int(slots), c_int(tokens), _stream())
+    return out
+
+
+_SCAN_SHAPES = ((4, 4), (8, 4), (16, 1), (16, 2), (16, 4), (16, 8), (16, 16))   # (lanes a channel, states a lane)
+SCAN_TARGET_BLOCKS = 512
+
+
+def scan_shape(channels: int, states: int, num_seqs: int) -> tuple[int, int]:
+    """How many lanes share a channel and how many states each holds: the fewest lanes whose launch still has
+    about two blocks a CU, else the most; then the fewest states a lane that hold them all."""
+    fitting = [(lanes, per) for lanes, per in _SCAN_SHAPES if lanes * per >= states]
+    if not fitting:
+        raise KernelError(f"up to 256 states a channel, not {states}")
+    by_lanes: dict[int, int] = {}
+    for lanes, per in fitting:
+        by_lanes[lanes] = min(per, by_lanes.get(lanes, per))
+    for lanes in sorted(by_lanes):
+        if -(-channels * lanes // 256) * num_seqs >= SCAN_TARGET_BLOCKS:
+            return lanes, by_lanes[lanes]
+    lanes = max(by_lanes)
+    return lanes, by_lanes[lanes]
+
+
+def selective_scan(x: Tensor, dt_lin: Tensor, dt_bias: Tensor, a: Tensor, bc: Tensor, d: Tensor, z: Tensor, state: Tensor,
+                   cu_q: Tensor, state_slots: Tensor, *, num_seqs: int) -> Tensor:
+    """The selective state-space recurrence, per sequence, channel c and state n, token after token:
+    ``dt = softplus(dt_lin[t, c] + dt_bias[c])``, ``S[c, n] <- exp(dt a[c, n]) S[c, n] + dt x[t, c] B[t, n]``,
+    ``y[t, c] = (sum_n S[c, n] C[t, n] + d[c] x[t, c]) * silu(z[t, c])``.  x [T, C]; dt_lin float32 [T, C];
+    dt_bias, d float32 [C]; a float32 [C, N] (negative); bc float32 [T, >= 2N] (B, then C) and z [T, >= C] with
+    any row stride; state float32 [slots, C, N], read at the step's start and written at its end.  Returns
+    [T, C] in x's dtype; everything inside is float32."""
+    _gpu(x, "x")
+    tokens, channels = x.shape
+    _gpu(dt_lin, "dt_lin", torch.float32)
+    _gpu(dt_bias, "dt_bias", torch.float32)
+    _gpu(a, "a", torch.float32)
+    _gpu(d, "d", torch.float32)
+    _gpu(bc, "bc", torch.float32, contiguous=False)
+    _gpu(z, "z", x.dtype, contiguous=False)
+    _gpu(state, "state", torch.float32)
+    if a.dim() != 2 or a.shape[0] != channels:
+        raise KernelError(f"a must be [{channels}, states]")
+    states = a.shape[1]
+    if dt_lin.shape != (tokens, channels) or dt_bias.shape != (channels,) or d.shape != (channels,):
+        raise KernelError("dt_lin must be [T, C], dt_bias and d [C]")
+    if state.dim() != 3 or state.shape[1:] != (channels, states):
+        raise KernelError(f"state must be [slots, {channels}, {states}], got {tuple(state.shape)}")
+    if bc.shape[0] != tokens or z.shape[0] != tokens:
+        raise KernelError("bc and z must have one row per token")
+    bc_stride = _strided_rows(bc, "bc", 2 * states)
+    z_stride = _strided_rows(z, "z", channels)
+    _sequences(cu_q, state_slots, num_seqs)
+    lanes, per_lane = scan_shape(channels, states, num_seqs)
+    out = torch.empty((tokens, channels), dtype=x.dtype, device=x.device)
+    _call("selective_scan", "fe_selective_scan", _ptr(x), c_int(_code(x.dtype)), _ptr(dt_lin), _ptr(dt_bias), _ptr(a), _ptr(bc),
+          c_longlong(bc_stride), _ptr(d), _ptr(z), c_longlong(z_stride), _ptr(state), _ptr(cu_q), _ptr(state_slots), _ptr(out),
+          c_int(tokens), c_int(num_seqs), c_int(channels), c_int(states), c_int(state.shape[0]), c_int(lanes), c_int(per_lane),
+          _stream())
     return out

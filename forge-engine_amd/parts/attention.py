@@ -22,7 +22,14 @@ one row per query head and the whole head is multiplied by that one number); ``w
 weight of that size, before the rotation); ``softcap`` (scores, after the scale, bounded as
 ``cap * tanh(score / cap)``); ``own_kv`` False (the layer has no k and v tensors at all and is only
 ever scheduled to read another call's cache); ``names`` (what the tensors are called in the
-checkpoint).  A position part may scale its cosines and sines (``magnitude``).  With any of them the step takes the general path:
+checkpoint); ``output_bias`` (whether the output projection has a bias; by default as ``bias`` says, False
+gives biases on q, k and v alone); ``fixed_sink`` (a number that joins every head's softmax as a
+score without key or value: 0 puts a one into the denominator); ``distance_slope_bits`` (c: head h's
+score of key j loses ``2^(-c (h + 1) / H) * (i - j)``, H heads, after the scale); ``value_mix``
+("source": the layer leaves its values of the step's tokens for later layers; "blend": its values
+become ``(1 - m) v + m v_source`` with m a scalar tensor of the layer, before they are cached);
+``force_general`` (take the general path whatever the options).  A position part may scale its
+cosines and sines (``magnitude``).  With any of them the step takes the general path:
 one product for q, k, v (and the gate), one kernel for convolution, rotation, norms and the
 page write, the masked attention kernel, the gate, the output projection.
 """
@@ -46,7 +53,9 @@ class GroupedQueryAttention(Mixer):
                  value_dim: int | None = None, conv_taps: int = 0, unit_norm_eps: float | None = None,
                  chunk: int | None = None, sink: bool = False, output_gate: bool = False,
                  head_gate: bool = False, whole_norm_eps: float | None = None, softcap: float | None = None,
-                 own_kv: bool = True, names: dict[str, str] | None = None) -> None:
+                 own_kv: bool = True, names: dict[str, str] | None = None, output_bias: bool | None = None,
+                 fixed_sink: float | None = None, distance_slope_bits: float | None = None,
+                 value_mix: str | None = None, value_mix_key: str = "values", force_general: bool = False) -> None:
         super().__init__(ctx, prefix)
         if num_heads % num_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")
@@ -71,6 +80,18 @@ class GroupedQueryAttention(Mixer):
         self.softcap = None if softcap is None else float(softcap)
         self.own_kv = own_kv
         self.gate_size = 0 if not self.output_gate else (num_heads if head_gate else self.out_size)
+        self.output_bias = bool(bias) if output_bias is None else bool(output_bias)
+        self.fixed_sink = None if fixed_sink is None else float(fixed_sink)
+        self.distance_slope_bits = None if distance_slope_bits is None else float(distance_slope_bits)
+        if value_mix not in (None, "source", "blend"):
+            raise ValueError(f"value_mix must be 'source' or 'blend', not {value_mix!r}")
+        if sink and fixed_sink is not None:
+            raise ValueError("a learned sink and a fixed one exclude each other")
+        if self.output_bias and not bias:
+            raise ValueError("a bias on the output projection comes with biases on q, k and v")
+        self.value_mix, self.value_mix_key = value_mix, value_mix_key
+        self.mix_weight: float | None = None
+        self.slopes: Tensor | None = None
         if whole_norm_eps is not None and (self.conv_taps or unit_norm_eps is not None or bias):
             raise ValueError("a norm over the whole projection is not combined with convolutions, unit norms or biases")
         if not own_kv and whole_norm_eps is None:
@@ -82,7 +103,11 @@ class GroupedQueryAttention(Mixer):
         # the general path: anything the fused kernels of the plain arrangement do not know
         self.general = bool(self.value_dim != head_dim or self.conv_taps or unit_norm_eps is not None
                             or chunk is not None or sink or self.output_gate or whole_norm_eps is not None
-                            or softcap is not None or not own_kv)
+                            or softcap is not None or not own_kv or fixed_sink is not None
+                            or distance_slope_bits is not None or value_mix is not None
+                            or self.output_bias != bool(bias) or force_general)
+        if (value_mix is not None or fixed_sink is not None or distance_slope_bits is not None) and whole_norm_eps is not None:
+            raise ValueError("value mixing, fixed sinks and distance slopes are not combined with the whole-projection norm")
         if self.general and qk_norm_eps is not None:
             raise ValueError("weighted q/k norms before the rotation are not combined with the general path's options")
         self.names = dict(self.DEFAULT_NAMES, **(names or {}))
@@ -116,7 +141,7 @@ class GroupedQueryAttention(Mixer):
         "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
         "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
         "q_conv": "q_proj.conv", "k_conv": "k_proj.conv", "v_conv": "v_proj.conv",
-        "sink": "sink", "gate": "gate_proj.weight",
+        "sink": "sink", "gate": "gate_proj.weight", "value_mix": "value_mix",
     }
 
     def param_specs(self):
@@ -133,10 +158,12 @@ class GroupedQueryAttention(Mixer):
             if self.own_kv:
                 specs[n["k_norm"]] = ParamSpec((self.kv_size,), kind="vector", init="norm")
         if self.bias:
-            specs[n["q_bias"]] = ParamSpec((self.q_size,), kind="vector", init="zeros")
-            specs[n["k_bias"]] = ParamSpec((self.kv_size,), kind="vector", init="zeros")
-            specs[n["v_bias"]] = ParamSpec((self.v_size,), kind="vector", init="zeros")
-            specs[n["o_bias"]] = ParamSpec((self.hidden_size,), kind="vector", init="zeros")
+            drawn = "small" if self.general else "zeros"      # random models of the general path get biases that show
+            specs[n["q_bias"]] = ParamSpec((self.q_size,), kind="vector", init=drawn)
+            specs[n["k_bias"]] = ParamSpec((self.kv_size,), kind="vector", init=drawn)
+            specs[n["v_bias"]] = ParamSpec((self.v_size,), kind="vector", init=drawn)
+            if self.output_bias:
+                specs[n["o_bias"]] = ParamSpec((self.hidden_size,), kind="vector", init="zeros")
         if self.qk_norm_eps is not None:
             specs[n["q_norm"]] = ParamSpec((self.head_dim,), kind="vector", init="norm")
             specs[n["k_norm"]] = ParamSpec((self.head_dim,), kind="vector", init="norm")
@@ -148,6 +175,8 @@ class GroupedQueryAttention(Mixer):
             specs[n["sink"]] = ParamSpec((self.num_heads,), kind="vector", init="unit")
         if self.output_gate:
             specs[n["gate"]] = ParamSpec((self.gate_size, self.hidden_size))
+        if self.value_mix is not None:      # a scalar; the source layer's is never read
+            specs[n["value_mix"]] = ParamSpec((), kind="vector", init="uniform", optional=self.value_mix == "source")
         return specs
 
     def set_param(self, name: str, tensor: Tensor) -> None:
@@ -182,10 +211,18 @@ class GroupedQueryAttention(Mixer):
             self.k_norm = tensor
         elif key == "sink":
             self.sink_weight = tensor
+        elif key == "value_mix" and self.value_mix is not None:
+            self.mix_weight = float(tensor.reshape(()).item())
         else:
             raise KeyError(name)
 
     def finalize(self) -> None:
+        device = self.qkv_weight.device
+        if self.fixed_sink is not None:
+            self.sink_weight = torch.full((self.num_heads,), self.fixed_sink, dtype=torch.float32, device=device)
+        if self.distance_slope_bits is not None:
+            slopes = [2.0 ** (-self.distance_slope_bits * (head + 1) / self.num_heads) for head in range(self.num_heads)]
+            self.slopes = torch.tensor(slopes, dtype=torch.float64).to(torch.float32).to(device)
         # the general path adds biases in float32 behind the products, which then take the kernels for few rows
         self.conv_bias = None if self.qkv_bias is None else self.qkv_bias[:self.conv_channels].float().contiguous()
         self.o_bias_f32 = None if self.o_bias is None else self.o_bias.float().contiguous()
@@ -273,19 +310,28 @@ class GroupedQueryAttention(Mixer):
             q, cache.key_pages, cache.value_pages, attn, batch.cu_q, batch.ctx_len, cache.block_table,
             num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim, scale=self.scale,
-            window=self.window, chunk=self.chunk, sink=self.sink_weight,
+            window=self.window, chunk=self.chunk, sink=self.sink_weight, slopes=self.slopes,
             gate=qkv[:, self.conv_channels:] if self.output_gate else None, num_decode=batch.num_decode,
             max_ctx=batch.max_ctx, softcap=self.softcap, head_gate=self.head_gate)
         update = ops.linear_update(attn, self.o_weight)
         return update if self.o_bias_f32 is None else ops.add_bias(update, self.o_bias_f32)
 
     def _conv_rope(self, qkv: Tensor, q: Tensor, batch, cache: CacheView, inv_freq, rotary_dim: int) -> None:
+        mixing = {}
+        if self.value_mix == "source":
+            kept = torch.empty((qkv.shape[0], self.v_size), dtype=qkv.dtype, device=qkv.device)
+            batch.carry[self.value_mix_key] = kept
+            mixing = {"v_keep": kept}
+        elif self.value_mix == "blend":
+            if self.value_mix_key not in batch.carry:
+                raise ValueError(f"{self.prefix}: no earlier layer of the step left the values '{self.value_mix_key}'")
+            mixing = {"v_from": batch.carry[self.value_mix_key], "v_mix": self.mix_weight}
         ops.conv_rope_norm_write(
             qkv, self.conv_bias, self.conv_weight, cache.states[self.CONV_STATE] if self.conv_taps > 1 else None, inv_freq,
             batch.positions, batch.token_seq, batch.cu_q, batch.state_slots, cache.block_table,
             cache.key_pages, cache.value_pages, q, num_seqs=batch.num_seqs, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim,
-            rotary_dim=rotary_dim, unit_norm_eps=self.unit_norm_eps, taps=self.conv_taps)
+            rotary_dim=rotary_dim, unit_norm_eps=self.unit_norm_eps, taps=self.conv_taps, **mixing)
 
     def _single_tokens_only(self, batch, x: Tensor, cache: CacheView, rotary_dim: int) -> bool:
         """Every sequence of the step brings one token, and the sizes are ones that the

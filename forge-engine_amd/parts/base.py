@@ -65,11 +65,26 @@ class Residual:
         self.pending: Tensor | None = None
         self.streams: Tensor | None = None
         self.pending_mix: tuple[Tensor, Tensor] | None = None    # (mix [S, S] indexed [from, to], share [S])
+        self.pending_norm: tuple[Tensor, float] | None = None    # (weight, eps): the update is RMS-normed before it is added
 
     def add(self, update: Tensor | None) -> None:
         """Leave an update pending; None: the part has added it into the stream itself."""
         self.flush()
         self.pending = update
+
+    def add_normed(self, update: Tensor, weight: Tensor, eps: float) -> None:
+        """Leave ``h += update * rsqrt(mean(update^2) + eps) * weight`` pending (a norm behind a
+        sublayer): the next norm's kernel applies it and normalises the new stream in one pass."""
+        self.flush()
+        if self.streams is not None:
+            raise ValueError("a norm behind a sublayer needs a model with one residual stream")
+        self.pending, self.pending_norm = update, (weight, float(eps))
+
+    def take_normed(self):
+        """(update, weight, eps) of a pending update that is to be normed, which the caller now applies."""
+        update, (weight, eps) = self.pending, self.pending_norm
+        self.pending = self.pending_norm = None
+        return update, weight, eps
 
     def add_mixed(self, update: Tensor, mix: Tensor, share: Tensor) -> None:
         """Several streams: leave ``x_t <- sum_s mix[s, t] x_s + share[t] * update`` pending."""
@@ -102,6 +117,9 @@ class Residual:
             if self.streams is not None:
                 update, mix, share = self.take_pending()
                 ops.hyper_norm(self.streams, update, mix, share, None, None, None, 0.0, None)
+            elif self.pending_norm is not None:
+                update, weight, eps = self.take_normed()
+                ops.rmsnorm_update(self.h, update, weight, eps, None)
             else:
                 ops.add_rows(self.h, self.pending)
                 self.pending = None

@@ -94,6 +94,29 @@ class OutputNormBlock(Block):
         return {"stream_ops"}
 
 
+class SandwichNormBlock(Block):
+    """A norm before and a norm behind each sublayer: ``h += norm_mb(mixer(norm_m(h)))``, then
+    ``h += norm_fb(ffn(norm_f(h)))``.  The norm behind a sublayer is left pending on the stream with
+    its update (``Residual.add_normed``), so that the kernel of the next norm before a sublayer (in
+    this layer, in the next one, or the model's last norm) applies both in one pass.  A layer may
+    have no feed-forward."""
+
+    NORMS = ("input", "mixer_out", "post_mixer", "ff_out")
+
+    def forward(self, residual: Residual, batch, cache: CacheView | None, writes_cache: bool = True) -> None:
+        x = self.norms["input"].forward(residual)
+        behind = self.norms["mixer_out"]
+        residual.add_normed(self.mixer.forward(x, batch, cache, writes_cache), behind.weight, behind.eps)
+        if self.feed_forward is None:
+            return
+        y = self.norms["post_mixer"].forward(residual)
+        behind = self.norms["ff_out"]
+        residual.add_normed(self.feed_forward.forward(y, batch), behind.weight, behind.eps)
+
+    def kernel_libraries(self):
+        return {"stream_ops"}
+
+
 class HyperConnectionBlock(Block):
     """Pre-norm sublayers over ``streams`` residual streams instead of one.  Sublayer q (the mixer,
     then the feed-forward) reads ``u = sum_s in_q[s] x_s``, computes ``y = sublayer(norm_q(u))``, and
@@ -155,4 +178,5 @@ class HyperConnectionBlock(Block):
 
 register_part("block", "hyper_connections", HyperConnectionBlock)
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("block", "output_norm", OutputNormBlock)

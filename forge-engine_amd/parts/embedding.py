@@ -19,11 +19,13 @@ from .base import BuildContext, Embedding, Head, ParamSpec, Residual
 
 class TokenEmbedding(Embedding):
     def __init__(self, ctx: BuildContext, prefix: str, *, vocab_size: int, hidden_size: int,
-                 leaf: str = "weight") -> None:
+                 leaf: str = "weight", scale: float = 1.0) -> None:
+        """``scale``: a factor on every row as it enters the float32 stream."""
         super().__init__(ctx, prefix)
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.leaf = leaf        # the table's name behind the prefix ("": the prefix itself)
+        self.scale = float(scale)
         self.weight: Tensor | None = None
 
     def param_specs(self):
@@ -37,10 +39,12 @@ class TokenEmbedding(Embedding):
     def forward(self, batch) -> Residual:
         h = torch.empty((batch.num_tokens, self.hidden_size), dtype=torch.float32, device=self.weight.device)
         ops.embed_rows(batch.token_ids, self.weight, h)
+        if self.scale != 1.0:
+            ops.scale_rows(h, self.scale)
         return Residual(h)
 
     def kernel_libraries(self):
-        return {"rowwise"}
+        return {"rowwise"} | ({"hyper"} if self.scale != 1.0 else set())
 
 
 class TokenPairEmbedding(TokenEmbedding):

@@ -97,5 +97,45 @@ class PolyNormMLP(FeedForward):
         return {"stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
 
 
+class ActivatedMLP(FeedForward):
+    """``down(act(up(x)))`` without a gate and without biases; ``activation``: ``relu_squared``
+    (``max(z, 0)^2``)."""
+
+    ACTIVATIONS = ("relu_squared",)
+
+    def __init__(self, ctx: BuildContext, prefix: str, *, hidden_size: int, intermediate_size: int,
+                 activation: str = "relu_squared", names: dict[str, str] | None = None) -> None:
+        super().__init__(ctx, prefix)
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"unknown activation '{activation}' (known: {', '.join(self.ACTIVATIONS)})")
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.activation = activation
+        self.names = dict({"up": "up", "down": "down"}, **(names or {}))
+        self.up_weight: Tensor | None = None
+        self.down_weight: Tensor | None = None
+
+    def param_specs(self):
+        inter, hidden = self.intermediate_size, self.hidden_size
+        return {self.name(self.names["up"]): ParamSpec((inter, hidden)),
+                self.name(self.names["down"]): ParamSpec((hidden, inter))}
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        if name == self.name(self.names["up"]):
+            self.up_weight = tensor
+        elif name == self.name(self.names["down"]):
+            self.down_weight = tensor
+        else:
+            raise KeyError(name)
+
+    def forward(self, x: Tensor, batch=None) -> Tensor:
+        act = ops.relu_squared(ops.linear(x, self.up_weight))
+        return ops.linear_update(act, self.down_weight)
+
+    def kernel_libraries(self):
+        return {"stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+
+
+register_part("feed_forward", "activated_mlp", ActivatedMLP)
 register_part("feed_forward", "swiglu", SwiGLU)
 register_part("feed_forward", "polynorm_mlp", PolyNormMLP)

@@ -7,6 +7,12 @@ their weights are the softmax over the chosen logits alone.  Expert (no biases):
 experts' outputs, plus a shared expert of the same form (sizes and limit of its own) that every
 token takes.
 
+Options: ``scoring`` "sigmoid" (a chosen expert's weight is the sigmoid of its own logit, not
+renormalised over the chosen); ``form`` "silu" (``y = W_down (silu(W_gate x) * (W_up x))``, no
+bounds); ``weight_input`` (the weight multiplies the expert's input, ``expert(w x)``, instead of
+its output; since the first products are linear, they are scaled behind their sums);
+``router_bias`` False (the router has no bias tensor).
+
 A step sorts its (token, choice) pairs by expert on the device and runs two grouped products over
 the sorted rows (gate and up with the activation as their ending, then down, weighted by the
 router); nothing is decided on the host, so steps are captured like any other.  The update comes
@@ -26,8 +32,9 @@ from .base import BuildContext, FeedForward, ParamSpec
 
 class RoutedExperts(FeedForward):
     def __init__(self, ctx: BuildContext, prefix: str, *, hidden_size: int, experts: int, top: int,
-                 intermediate_size: int, limit: float, alpha: float = 1.702, shared_size: int | None = None,
-                 shared_limit: float | None = None, names: dict[str, str] | None = None) -> None:
+                 intermediate_size: int, limit: float | None = None, alpha: float = 1.702, shared_size: int | None = None,
+                 shared_limit: float | None = None, names: dict[str, str] | None = None, scoring: str = "softmax",
+                 form: str = "bounded", weight_input: bool = False, router_bias: bool = True) -> None:
         """``names``: what the tensors are called behind the prefix; ``expert`` is a pattern with
         ``{e}`` for the expert's number."""
         super().__init__(ctx, prefix)
@@ -38,9 +45,14 @@ class RoutedExperts(FeedForward):
         self.hidden_size = hidden_size
         self.experts, self.top = experts, top
         self.intermediate_size = intermediate_size
-        self.limit, self.alpha = float(limit), float(alpha)
+        if scoring not in ("softmax", "sigmoid") or form not in ("bounded", "silu"):
+            raise ValueError(f"unknown scoring '{scoring}' or form '{form}'")
+        if form == "bounded" and limit is None:
+            raise ValueError("the bounded activation needs a limit")
+        self.scoring, self.form, self.weight_input, self.has_router_bias = scoring, form, bool(weight_input), bool(router_bias)
+        self.limit, self.alpha = float(limit or 0.0), float(alpha)
         self.shared_size = shared_size
-        self.shared_limit = float(limit if shared_limit is None else shared_limit)
+        self.shared_limit = float(self.limit if shared_limit is None else shared_limit)
         self.names = dict({"expert": "experts.{e}", "shared": "shared", "router": "router.weight", "router_bias": "router.bias",
                            "gate": "gate", "up": "up", "down": "down"}, **(names or {}))
         self.router_weight: Tensor | None = None
@@ -56,8 +68,9 @@ class RoutedExperts(FeedForward):
 
     def param_specs(self):
         f, h = self.intermediate_size, self.hidden_size
-        specs = {self.name(self.names["router"]): ParamSpec((self.experts, h), init="router"),
-                 self.name(self.names["router_bias"]): ParamSpec((self.experts,), kind="vector", init="small")}
+        specs = {self.name(self.names["router"]): ParamSpec((self.experts, h), init="router")}
+        if self.has_router_bias:
+            specs[self.name(self.names["router_bias"])] = ParamSpec((self.experts,), kind="vector", init="small")
         for expert in range(self.experts):
             specs[self._expert_name(expert, "gate")] = ParamSpec((f, h))
             specs[self._expert_name(expert, "up")] = ParamSpec((f, h))
@@ -77,7 +90,7 @@ class RoutedExperts(FeedForward):
         if name == self.name(self.names["router"]):
             self.router_weight = tensor.contiguous()
             return
-        if name == self.name(self.names["router_bias"]):
+        if self.has_router_bias and name == self.name(self.names["router_bias"]):
             self.router_bias = tensor.contiguous()
             return
         if not hasattr(self, "_owners"):
@@ -110,17 +123,20 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x: Tensor, batch=None) -> Tensor:
         tokens = x.shape[0]
-        chosen, weights = ops.moe_route(x, self.router_weight, self.router_bias, self.top)
+        chosen, weights = ops.moe_route(x, self.router_weight, self.router_bias, self.top, self.scoring)
         shared = None
         if self.shared_size:
-            act = ops.linear_gated(x, self.shared_gate_up, limit=self.shared_limit, alpha=self.alpha)
+            if self.form == "silu":     # the gated SiLU of the dense feed-forward, with its fused kernels
+                act = ops.linear_swiglu(x, self.shared_gate_up)
+            else:
+                act = ops.linear_gated(x, self.shared_gate_up, limit=self.shared_limit, alpha=self.alpha)
             shared = ops.linear_update(act, self.shared_down)
         update = torch.empty((self.top, tokens, self.hidden_size), dtype=torch.float32, device=x.device)
         return ops.moe_experts(x, chosen, weights, self.gate_up, self.down, update, limit=self.limit, alpha=self.alpha,
-                               extra=shared)
+                               extra=shared, form=self.form, weight_input=self.weight_input)
 
     def kernel_libraries(self):
-        return {"moe", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+        return {"moe", "rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "gemm_tile"}
 
 
 register_part("feed_forward", "routed_experts", RoutedExperts)

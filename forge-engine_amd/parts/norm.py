@@ -17,23 +17,29 @@ from .base import BuildContext, Norm, ParamSpec, Residual
 
 
 class RMSNorm(Norm):
-    def __init__(self, ctx: BuildContext, prefix: str, *, size: int, eps: float, leaf: str = "weight") -> None:
-        """``leaf``: the weight's name behind the prefix ("": the prefix itself is the name)."""
+    def __init__(self, ctx: BuildContext, prefix: str, *, size: int, eps: float, leaf: str = "weight",
+                 offset: float = 0.0) -> None:
+        """``leaf``: the weight's name behind the prefix ("": the prefix itself is the name).
+        ``offset``: what the stored weight is the distance from (1: weights stored around zero,
+        applied as ``1 + w``; the sum is formed once, in float32, when the tensor is loaded)."""
         super().__init__(ctx, prefix)
         self.size = size
         self.eps = float(eps)
         self.leaf = leaf
+        self.offset = float(offset)
         self.weight: Tensor | None = None
 
     def param_specs(self):
-        return {self.name(self.leaf): ParamSpec((self.size,), kind="vector", init="norm")}
+        return {self.name(self.leaf): ParamSpec((self.size,), kind="vector", init="small" if self.offset else "norm")}
 
     def set_param(self, name: str, tensor: Tensor) -> None:
         if name != self.name(self.leaf):
             raise KeyError(name)
-        self.weight = tensor
+        self.weight = tensor + self.offset if self.offset else tensor
 
     def forward(self, residual: Residual, rows: Tensor | None = None) -> Tensor:
+        if residual.pending_norm is not None:    # a normed update: into the stream first
+            residual.flush()
         if rows is not None:    # the chosen rows of stream + pending update; both are left as they are
             h = residual.h
             out = torch.empty((rows.numel(), self.size), dtype=self.ctx.dtype, device=h.device)

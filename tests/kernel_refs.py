@@ -370,7 +370,7 @@ def add_bias(update, bias):
 
 def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, block_table,
                          key_pages, value_pages, q_out, *, num_seqs, q_heads, kv_heads, head_dim, value_dim, rotary_dim,
-                         unit_norm_eps, taps):
+                         unit_norm_eps, taps, v_from=None, v_mix=0.0, v_keep=None):
     tokens = qkv.shape[0]
     q_size, k_size, v_size = q_heads * head_dim, kv_heads * head_dim, kv_heads * value_dim
     channels = q_size + k_size + v_size
@@ -404,7 +404,12 @@ def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions
 
     q = rotate_norm(y[:, :q_size].view(tokens, q_heads, head_dim))
     k = rotate_norm(y[:, q_size:q_size + k_size].view(tokens, kv_heads, head_dim)).to(qkv.dtype)
-    v = y[:, q_size + k_size:].view(tokens, kv_heads, value_dim).to(qkv.dtype)
+    v = y[:, q_size + k_size:]
+    if v_from is not None:
+        v = (1.0 - v_mix) * v + v_mix * v_from.float()
+    v = v.view(tokens, kv_heads, value_dim).to(qkv.dtype)
+    if v_keep is not None:
+        v_keep.copy_(v.reshape(tokens, v_size))
     q_out.copy_(q.reshape(tokens, q_size).to(q_out.dtype))
     block_size = key_pages.shape[2]
     for t in range(tokens):
@@ -417,7 +422,7 @@ def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions
 
 def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, q_heads, kv_heads,
                      head_dim, value_dim, scale, window=None, chunk=None, sink=None, gate=None, num_decode=None, max_ctx=None,
-                     softcap=None, head_gate=False):
+                     softcap=None, head_gate=False, slopes=None):
     block_size = key_pages.shape[2]
     groups = q_heads // kv_heads
     for s in range(num_seqs):
@@ -440,6 +445,8 @@ def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table,
                 scores = (keys[g, first:p + 1] @ qv) * scale
                 if softcap is not None:
                     scores = softcap * torch.tanh(scores / softcap)
+                if slopes is not None:
+                    scores = scores - slopes[h] * (p - torch.arange(first, p + 1, device=scores.device)).float()
                 top = scores.max()
                 if sink is not None:
                     top = torch.maximum(top, sink[h])
@@ -586,27 +593,32 @@ def whole_norm_rope_write(qkv, q_weight, k_weight, inv_freq, positions, token_se
         value_pages[page, :, :, pos % block_size] = v[t]
 
 
-def moe_route(x, router_weight, router_bias, top):
+def moe_route(x, router_weight, router_bias, top, scoring="softmax"):
     z = x.float() @ router_weight.float().T
     if router_bias is not None:
         z = z + router_bias
     best = torch.topk(z, top, dim=-1)
-    return best.indices.to(torch.int32), torch.softmax(best.values, dim=-1)
+    weights = torch.sigmoid(best.values) if scoring == "sigmoid" else torch.softmax(best.values, dim=-1)
+    return best.indices.to(torch.int32), weights
 
 
-def _gated(g, u, limit, alpha):
+def _gated(g, u, limit, alpha, form="bounded"):
+    if form == "silu":
+        return g * torch.sigmoid(g) * u
     g = g.clamp(max=limit)
     return g * torch.sigmoid(alpha * g) * (u.clamp(-limit, limit) + 1.0)
 
 
-def moe_experts(x, chosen, weights, gate_up, down, out, *, limit, alpha, extra=None):
+def moe_experts(x, chosen, weights, gate_up, down, out, *, limit=0.0, alpha=1.0, extra=None, form="bounded", weight_input=False):
     inner = gate_up.shape[1] // 2
     for t in range(x.shape[0]):
         for k in range(chosen.shape[1]):
             e = int(chosen[t, k])
             gu = gate_up[e].float() @ x[t].float()
-            act = _gated(gu[:inner], gu[inner:], limit, alpha).to(x.dtype).float()
-            out[k, t] = weights[t, k] * (down[e].float() @ act)
+            if weight_input:
+                gu = gu * weights[t, k]
+            act = _gated(gu[:inner], gu[inner:], limit, alpha, form).to(x.dtype).float()
+            out[k, t] = (1.0 if weight_input else weights[t, k]) * (down[e].float() @ act)
     if extra is not None:
         out[0] += _sum_parts(extra)
     return out
@@ -616,6 +628,53 @@ def linear_gated(x, gate_up_weight, *, limit, alpha):
     gu = linear(x, gate_up_weight).float()
     inner = gu.shape[1] // 2
     return _gated(gu[:, :inner], gu[:, inner:], limit, alpha).to(x.dtype)
+
+
+def relu_squared(x):
+    return torch.relu(x.float()).square().to(x.dtype)
+
+
+def causal_conv_act(u, weight, bias, state, token_seq, cu_q, state_slots, *, num_seqs, act="silu"):
+    channels, taps = weight.shape
+    rows = u[:, :channels].float()
+    out = torch.empty((u.shape[0], channels), dtype=u.dtype, device=u.device)
+    for s in range(num_seqs):
+        a, b = int(cu_q[s]), int(cu_q[s + 1])
+        if b == a:
+            continue
+        if taps > 1:
+            slot = int(state_slots[s])
+            history = torch.cat([state[slot], rows[a:b]])
+            state[slot] = history[-(taps - 1):]
+        else:
+            history = rows[a:b]
+        y = sum(history[j:j + b - a] * weight[:, j] for j in range(taps))
+        if bias is not None:
+            y = y + bias
+        if act == "silu":
+            y = y * torch.sigmoid(y)
+        out[a:b] = y.to(out.dtype)
+    return out
+
+
+def selective_scan(x, dt_lin, dt_bias, a, bc, d, z, state, cu_q, state_slots, *, num_seqs):
+    channels, states = a.shape
+    out = torch.empty_like(x)
+    dt = torch.nn.functional.softplus((dt_lin + dt_bias).double())
+    for s in range(num_seqs):
+        lo, hi = int(cu_q[s]), int(cu_q[s + 1])
+        if hi == lo:
+            continue
+        slot = int(state_slots[s])
+        memory = state[slot].double()
+        for t in range(lo, hi):
+            xt = x[t].double()
+            memory = torch.exp(dt[t][:, None] * a.double()) * memory + (dt[t] * xt)[:, None] * bc[t, :states].double()[None, :]
+            y = memory @ bc[t, states:2 * states].double() + d.double() * xt
+            zt = z[t, :channels].double()
+            out[t] = (y * zt * torch.sigmoid(zt)).to(out.dtype)
+        state[slot] = memory.float()
+    return out
 
 
 def decode_prepare_supported(*args, **kwargs):
@@ -635,7 +694,8 @@ NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsno
          "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_filtered_rows",
          "cast_rows", "add_bias", "token_shift", "rmsnorm_update", "rmsnorm_mean", "polynorm", "tanh_rows", "head_norm_gate",
          "conv_rope_norm_write", "masked_attention", "linear_recurrence", "mlstm_gate_scan",
-         "hyper_norm", "embed_token_pairs", "scale_rows", "whole_norm_rope_write", "moe_route", "moe_experts", "linear_gated")
+         "hyper_norm", "embed_token_pairs", "scale_rows", "whole_norm_rope_write", "moe_route", "moe_experts", "linear_gated",
+         "relu_squared", "causal_conv_act", "selective_scan")
 
 
 def install(monkeypatch):
