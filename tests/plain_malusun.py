@@ -133,7 +133,7 @@ def attention_mixer(h, w, p, sizes, positions, kind: str, shared: dict, cache: d
     if sizes.get("v_mix"):
         if "v_first" in shared:
             lam = w[p + ".vmix"]
-            v = (1.0 - lam) * v + lam * shared["v_first"]
+            v = (1.0 - lam) * v + lam * shared["v_first"].reshape(v.shape)    # heads side by side, if they are cut differently
         else:
             shared["v_first"] = v
     k_positions = positions
@@ -162,12 +162,14 @@ def expert_mixture(h, w, p, mlp: dict, margins: list | None = None) -> torch.Ten
     experts, top = mlp["router"]["experts"], mlp["router"]["top"]
     scores = torch.sigmoid(h @ w[p + ".router"].T)
     out = torch.zeros_like(h)
+    gaps = []
     for t in range(h.shape[0]):
         order = sorted(range(experts), key=lambda e: (-float(scores[t, e]), e))
-        if margins is not None and top < experts:
-            margins.append(float(scores[t, order[top - 1]] - scores[t, order[top]]))
+        gaps.append(float(scores[t, order[top - 1]] - scores[t, order[top]]) if top < experts else 1.0)
         for e in order[:top]:
             out[t] += gated_expert(scores[t, e] * h[t], w, f"{p}.e{e}")
+    if margins is not None:     # per token: by how much the last chosen score leads the first one left out
+        margins.append(torch.tensor(gaps, dtype=F64))
     if mlp.get("shared") is not None:
         out = out + gated_expert(h, w, p + ".shared")
     return out
