@@ -387,7 +387,9 @@ class ModelRunner:
         cache.commit_single_tokens(records)
         self.steps_run += 1
         if not any(group.gives_back for group in cache.groups):   # a window gives pages back as it moves
-            room = min(len(table) * self.block_size - record.length for record in records for table in record.tables)
+            # (a model without keys and values in pages has no tables: its requests never run out of room)
+            room = min((len(table) * self.block_size - record.length for record in records for table in record.tables),
+                       default=1 << 30)
             self._steady = _SteadyDecode(tuple(e.request_id for e in entries), records, slot, room)
         return slot.logits
 
