@@ -112,7 +112,7 @@ def parse_args():
     parser.add_argument("--points", default=None, help="other decode batch sizes to report")
     parser.add_argument("--widths", default="1024,2048,4096",
                         help="--phase design: model widths at which Mazanex and Qwen3 are measured side by side")
-    parser.add_argument("--design", choices=("mazanex", "rekezen"), default="mazanex",
+    parser.add_argument("--design", choices=("mazanex", "rekezen", "malusun"), default="mazanex",
                         help="--phase design: which design is measured beside Qwen3")
     parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro", "check", "design"), default="all",
                         help="run one phase only (for profiles); the record then holds that phase alone")
@@ -331,8 +331,31 @@ def rekezen_configs(width: int, layers: int) -> dict:
     return {"Rekezen": rekezen, "Qwen3": design_configs(width, layers)["Qwen3"]}
 
 
+def malusun_configs(width: int, layers: int) -> dict:
+    """Malusun beside Rekezen (the closest existing model: attention over the general path and a mixture of experts
+    beside a shared one) and Qwen3, at one width: heads of 128 in groups of four, the same vocabulary and layer
+    count.  Malusun cycles through its three mixers: the selective scan (twice the width inside, 16 states a
+    channel, a step size of rank width / 16, four taps) with the dense feed-forward of three widths, then rotary
+    and penalised attention over windows of 1,024 with eight experts as wide as the model of which a token takes
+    two, beside a shared one of the same size; values lean on the first attention layer's."""
+    heads = max(4, width // 128)
+    attention = {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
+                 "v_mix": True}
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": width}, "shared": {"ff": width}}
+    kinds = [("mamba1", {"inner": 2 * width, "state": 16, "dt_rank": max(8, width // 16), "conv": 4}, {"kind": "dense", "ff": 3 * width}),
+             ("attention", dict(attention, rot={"dims": 64, "base": 500000.0}), moe),
+             ("attention_2", attention, moe)]
+    malusun = {"architecture": "Malusun", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 0.5},
+               "layers": [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": kinds[i % 3][2]} for i in range(layers)]}
+    others = rekezen_configs(width, layers)
+    return {"Malusun": malusun, "Rekezen": others["Rekezen"], "Qwen3": others["Qwen3"]}
+
+
+DESIGN_CONFIGS = {"mazanex": design_configs, "rekezen": rekezen_configs, "malusun": malusun_configs}
+
+
 def design_comparison(args) -> int:
-    """Prefill and decode throughput of Mazanex (or, with ``--design rekezen``, Rekezen) beside Qwen3 (the closest existing model) at equal
+    """Prefill and decode throughput of Mazanex (or, with ``--design``, Rekezen or Malusun) beside the closest existing models at equal
     width, layer count, feed-forward size and vocabulary; random weights, one JSON line a model and width."""
     import torch
 
@@ -346,7 +369,7 @@ def design_comparison(args) -> int:
     prompt_len = args.prompt_len or 1024
     generator = torch.Generator().manual_seed(args.seed)
     for width in (int(w) for w in args.widths.split(",")):
-        for label, raw in (rekezen_configs if args.design == "rekezen" else design_configs)(width, layers).items():
+        for label, raw in DESIGN_CONFIGS[args.design](width, layers).items():
             config = load_model_config(raw)
             model = random_model(config, args.seed, dtype=dtype, device=device)
             pages = -(-(max(args.prefill_tokens, prompt_len) + args.steps + args.warmup + 16) // args.block_size)

@@ -133,13 +133,14 @@ __device__ __forceinline__ int wave_most(int v) {
   return __builtin_amdgcn_readfirstlane(max((int)r[0], (int)r[1]));
 }
 
-template <int D, int KG, int RM, bool CAP = false>
+template <int D, int KG, int RM, bool CAP = false, bool SLOPE = false>
 __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_kernel(   // RM = 1: four waves a SIMD (128 registers), RM = 2: two
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int block_shift, int num_blocks, int window,
-    float scale_log2, int num_seqs, int heads_per_xcd, int chunk, const float* __restrict__ sink, float cap_ratio) {
+    float scale_log2, int num_seqs, int heads_per_xcd, int chunk, const float* __restrict__ sink, float cap_ratio,
+    const float* __restrict__ slopes) {
   const int block_mask = (1 << block_shift) - 1;
   constexpr int BM = 64 * RM;
   constexpr int KC = D / 32;            // MFMA k-steps over the head dim (scores)
@@ -378,8 +379,22 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
         st[rm][j >> 3][(j >> 2) & 1][j & 3] = cap_ratio * (1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(v * to_exponent) + 1.f));
       }
   };
+  // SLOPE: a penalty on distance, slope_h * (position - key), comes off the score after the scale: off the raw
+  // score it is that times 1 / scale (what it does to keys that the masks hide does not matter).
+  float slope_raw = 0.f;
+  if constexpr (SLOPE) slope_raw = slopes[head] * 1.4426950408889634f / scale_log2;
+  auto slope_scores = [&](int key_base, floatx4 (&st)[RM][2][2]) {
+#pragma unroll
+    for (int rm = 0; rm < RM; ++rm) {
+      const float nearest = (float)(row_pos[rm] - key_base - 8 * lq);     // the distance of the lane's first key of the tile
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        st[rm][j >> 3][(j >> 2) & 1][j & 3] -= slope_raw * (nearest - (float)(32 * (j >> 3) + (j & 7)));
+    }
+  };
   auto softmax = [&](int key_base, floatx4 (&st)[RM][2][2], uintx4 (&pw)[RM][2]) {
     if constexpr (CAP) cap_scores(st);
+    if constexpr (SLOPE) slope_scores(key_base, st);
     if (is_edge(key_base)) mask_edges(key_base, st);
 #pragma unroll
     for (int rm = 0; rm < RM; ++rm)
@@ -649,6 +664,11 @@ extern "C" int fe_paged_attention_prefill_masked(const void* q, long long q_stri
                                                  int groups, int head_dim, int block_size, int num_blocks,
                                                  int window, int chunk, const float* sink, float scale, int key_groups,
                                                  int row_sets, int total_q, hipStream_t stream);
+static int launch_prefill_sloped(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
+                                 long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
+                                 int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
+                                 int block_size, int num_blocks, int window, int chunk, const float* sink, float scale,
+                                 float softcap, const float* slopes, int key_groups, int row_sets, int total_q, hipStream_t stream);
 static int launch_prefill(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
                           long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
                           int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
@@ -697,13 +717,38 @@ extern "C" int fe_paged_attention_prefill_capped(const void* q, long long q_stri
                         scale, softcap, key_groups, row_sets, total_q, stream);
 }
 
+// The same with a penalty on distance: head h's score of key j, after the scale, loses slopes[h] * (position - j)
+// (slopes: float32 [kv_heads * groups]).
+extern "C" int fe_paged_attention_prefill_sloped(const void* q, long long q_stride, const void* key_pages,
+                                                 const void* value_pages, void* out, long long out_stride,
+                                                 const int* cu_q, const int* ctx_len, const int* block_table,
+                                                 int table_stride, int num_seqs, int max_q_len, int kv_heads,
+                                                 int groups, int head_dim, int block_size, int num_blocks,
+                                                 int window, int chunk, const float* sink, const float* slopes, float scale,
+                                                 int key_groups, int row_sets, int total_q, hipStream_t stream) {
+  if (!slopes || !(scale > 0.f)) return FE_BAD_ARGUMENT;
+  return launch_prefill_sloped(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len, block_table, table_stride,
+                               num_seqs, max_q_len, kv_heads, groups, head_dim, block_size, num_blocks, window, chunk, sink,
+                               scale, 0.f, slopes, key_groups, row_sets, total_q, stream);
+}
+
 static int launch_prefill(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
                           long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
                           int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
                           int block_size, int num_blocks, int window, int chunk, const float* sink, float scale,
                           float softcap, int key_groups, int row_sets, int total_q, hipStream_t stream) {
+  return launch_prefill_sloped(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len, block_table, table_stride,
+                               num_seqs, max_q_len, kv_heads, groups, head_dim, block_size, num_blocks, window, chunk, sink,
+                               scale, softcap, nullptr, key_groups, row_sets, total_q, stream);
+}
+
+static int launch_prefill_sloped(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
+                                 long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
+                                 int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
+                                 int block_size, int num_blocks, int window, int chunk, const float* sink, float scale,
+                                 float softcap, const float* slopes, int key_groups, int row_sets, int total_q, hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
-  if (chunk < 0) return FE_BAD_ARGUMENT;
+  if (chunk < 0 || (slopes && softcap > 0.f)) return FE_BAD_ARGUMENT;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
   if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
   if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1 || q_stride % 8 || out_stride % 4) return FE_BAD_ARGUMENT;
@@ -737,14 +782,15 @@ static int launch_prefill(const void* q, long long q_stride, const void* key_pag
   // least two tiles.
   if (key_groups == 0) key_groups = (row_sets == 1 && (long long)heads * filled_of(64) <= KEY_GROUPS_MAX_BLOCKS && max_q_len >= 128) ? 2 : 1;
   const float cap_ratio = softcap > 0.f ? softcap / scale : 0.f;
-#define FE_GO_C(DD, GG, RR, CC)                                                                                      \
-  paged_prefill_kernel<DD, GG, RR, CC><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+#define FE_GO_C(DD, GG, RR, CC, SS)                                                                                  \
+  paged_prefill_kernel<DD, GG, RR, CC, SS><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
-      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd, chunk, sink, cap_ratio)
-#define FE_GO(DD, GG, RR)                          \
-  do {                                             \
-    if (softcap > 0.f) FE_GO_C(DD, GG, RR, true);  \
-    else FE_GO_C(DD, GG, RR, false);               \
+      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd, chunk, sink, cap_ratio, slopes)
+#define FE_GO(DD, GG, RR)                                 \
+  do {                                                    \
+    if (softcap > 0.f) FE_GO_C(DD, GG, RR, true, false);  \
+    else if (slopes) FE_GO_C(DD, GG, RR, false, true);    \
+    else FE_GO_C(DD, GG, RR, false, false);               \
   } while (0)
 #define FE_GO_D(DD)                                          \
   if (key_groups == 1 && row_sets == 1) FE_GO(DD, 1, 1);      \

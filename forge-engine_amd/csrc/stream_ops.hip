@@ -146,6 +146,68 @@ extern "C" int fe_rmsnorm_update(float* h, const float* update, int parts, long 
   return fe_check_launch();
 }
 
+// A norm behind a sublayer and the norm before the next one in one pass over the row:
+//   v = h[s] + u * rsqrt(mean(u^2) + eps) * w        (u = the sum of the update's parts; written back to h if `store`)
+//   out[r] = v * rsqrt(mean(v^2) + eps_next) * w_next,  s = rows[r] or r.
+// The row (up to 8 elements a thread) stays in registers between the three passes.
+template <typename TO>
+__global__ __launch_bounds__(ROW_THREADS_FEW) void rmsnorm_update_norm_kernel(
+    float* __restrict__ h, const float* __restrict__ update, int parts, size_t part_stride,
+    const float* __restrict__ w, float eps, const float* __restrict__ w_next, float eps_next, TO* __restrict__ out,
+    const int* __restrict__ rows, int store, int width) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)(rows ? rows[blockIdx.x] : (int)blockIdx.x) * width;
+  const size_t out_base = (size_t)blockIdx.x * width;
+  const int threads = blockDim.x;
+  float u[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int c = threadIdx.x + j * threads;
+    u[j] = c < width ? parts_sum(update + base + c, parts, part_stride) : 0.f;
+    ss += u[j] * u[j];
+  }
+  ss = block_sum<true>(ss, scratch);
+  const float inv = rsqrtf(ss / (float)width + eps);
+  float ss_next = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int c = threadIdx.x + j * threads;
+    if (c < width) {
+      u[j] = h[base + c] + u[j] * inv * w[c];
+      if (store) h[base + c] = u[j];
+      ss_next += u[j] * u[j];
+    }
+  }
+  ss_next = block_sum(ss_next, scratch);
+  const float inv_next = rsqrtf(ss_next / (float)width + eps_next);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int c = threadIdx.x + j * threads;
+    if (c < width) store_from_float(out + out_base + c, u[j] * inv_next * w_next[c]);
+  }
+}
+
+// rows: indices of the rows to take (int32 [count]) or null for all `count` rows in order; with a row list
+// nothing is written back (store must be 0: rows may repeat).  Rows up to 8,192 wide (8 elements a thread).
+extern "C" int fe_rmsnorm_update_norm(float* h, const float* update, int parts, long long part_stride, const float* w,
+                                      float eps, const float* w_next, float eps_next, void* out, int out_dtype,
+                                      const int* rows, int store, int count, int width, hipStream_t stream) {
+  if (count <= 0) return FE_OK;
+  const int threads = width > 8 * ROW_THREADS ? ROW_THREADS_FEW : row_threads(count, width);
+  if (width <= 0 || width > 8 * threads || parts < 1 || parts > 64 || !(eps > 0.f) || !(eps_next > 0.f) || !out ||
+      (rows && store))
+    return FE_BAD_ARGUMENT;
+  if (out_dtype == FE_F32)
+    rmsnorm_update_norm_kernel<float><<<count, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, w_next,
+                                                                     eps_next, (float*)out, rows, store, width);
+  else if (out_dtype == FE_BF16)
+    rmsnorm_update_norm_kernel<bf16_t><<<count, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, w_next,
+                                                                      eps_next, (bf16_t*)out, rows, store, width);
+  else return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
 // out[r] = (1 / n) sum_b u_b * rsqrt(mean(u_b^2) + eps) * w[b]
 struct MeanInputs {
   const float* u[4];

@@ -714,12 +714,13 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
                     window: int | None = None, num_decode: int | None = None,
                     max_ctx: int | None = None, splits: int | None = None, chunk: int | None = None,
-                    sink: Tensor | None = None, softcap: float | None = None) -> Tensor:
+                    sink: Tensor | None = None, softcap: float | None = None, slopes: Tensor | None = None) -> Tensor:
     """Attention of every query token of a mixed batch over its paged keys.
 
     ``chunk`` (a token reads keys of its own run of that many positions only), ``sink``
-    (float32 [Hq]: exp(sink_h) joins head h's softmax denominator) and ``softcap`` (scores, after
-    the scale, become cap * tanh(score / cap)) are served by the two
+    (float32 [Hq]: exp(sink_h) joins head h's softmax denominator), ``softcap`` (scores, after
+    the scale, become cap * tanh(score / cap)) and ``slopes`` (float32 [Hq]: head h's score of key j
+    loses slopes[h] * (position - j); not together with a cap) are served by the two
     matrix-core kernels alone: a call that brings either for sizes those do not take is refused
     (``masked_attention`` routes such sizes to the vector-ALU kernel that knows both).
 
@@ -765,8 +766,12 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                   and q.data_ptr() % 16 == 0 and q_stride % 8 == 0)      # the fast kernels read 16 bytes at a time
     fast_decode = bf16_pages and head_dim in (64, 128, 256) and groups <= 8
     fast_prefill = bf16_pages and head_dim in (64, 128)
-    masked = chunk is not None or sink is not None or softcap is not None
+    masked = chunk is not None or sink is not None or softcap is not None or slopes is not None
     if masked:
+        if slopes is not None:
+            _gpu(slopes, "slopes", torch.float32)
+            if slopes.shape != (q_heads,) or softcap is not None or not scale > 0.0:
+                raise KernelError(f"slopes must be [{q_heads}], with a positive scale and without a soft cap")
         if (any_single and not fast_decode) or (any_longer and not fast_prefill):
             raise KernelError("chunks, sinks and soft caps are served by the matrix-core attention kernels only")
         if softcap is not None and not (softcap > 0.0 and scale > 0.0):
@@ -801,18 +806,20 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
             part_o = torch.empty(num_seqs * kv_heads * splits * groups * head_dim, dtype=torch.float32, device=q.device)
             part_ml = torch.empty(num_seqs * kv_heads * splits * groups * 2, dtype=torch.float32, device=q.device)
             counters = _split_counters(q.device, num_seqs * kv_heads)
-        mask = (c_int(chunk or 0), _ptr(sink)) if masked else ()
+        mask = (c_int(chunk or 0), _ptr(sink)) + ((_ptr(slopes),) if slopes is not None else ()) if masked else ()
         cap = (c_float(softcap),) if softcap is not None else ()
-        name = "fe_paged_attention_decode_capped" if cap else "fe_paged_attention_decode_masked" if masked else "fe_paged_attention_decode"
+        name = ("fe_paged_attention_decode_sloped" if slopes is not None else "fe_paged_attention_decode_capped" if cap
+                else "fe_paged_attention_decode_masked" if masked else "fe_paged_attention_decode")
         _call("attention_decode", name, _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(part_o),
               _ptr(part_ml), _ptr(counters), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
               c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
               c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), *cap, c_int(splits), _stream())
     if any_longer and fast_prefill:
-        mask = (c_int(chunk or 0), _ptr(sink)) if masked else ()
+        mask = (c_int(chunk or 0), _ptr(sink)) + ((_ptr(slopes),) if slopes is not None else ()) if masked else ()
         cap = (c_float(softcap),) if softcap is not None else ()
-        name = "fe_paged_attention_prefill_capped" if cap else "fe_paged_attention_prefill_masked" if masked else "fe_paged_attention_prefill"
+        name = ("fe_paged_attention_prefill_sloped" if slopes is not None else "fe_paged_attention_prefill_capped" if cap
+                else "fe_paged_attention_prefill_masked" if masked else "fe_paged_attention_prefill")
         _call("attention_prefill", name, _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
@@ -1078,6 +1085,43 @@ def rmsnorm_update(h: Tensor, update: Tensor, weight: Tensor, eps: float, out: T
     return out
 
 
+FUSED_NORMS_MAX_WIDTH = 8192       # 8 elements a thread at 1,024 threads a row
+
+
+def rmsnorm_update_norm(h: Tensor, update: Tensor, weight: Tensor, eps: float, next_weight: Tensor, next_eps: float, out: Tensor,
+                        rows: Tensor | None = None) -> Tensor:
+    """A norm behind a sublayer and the norm before the next one: ``v = h[s] + u * rsqrt(mean(u^2) + eps) * weight``
+    (u the update, float32, [parts, T, W] added up in order first), ``out[r] = v * rsqrt(mean(v^2) + next_eps) *
+    next_weight``, s = rows[r] or r; all float32 with one rounding at the store.  Without ``rows`` v is written back to
+    h; with them h stays as it is.  One kernel for rows up to FUSED_NORMS_MAX_WIDTH wide, two otherwise."""
+    _gpu(h, "h", torch.float32)
+    _gpu(weight, "weight", torch.float32)
+    _gpu(next_weight, "next_weight", torch.float32)
+    _gpu(out, "out")
+    total, width = h.shape
+    parts = _parts_of(update, total, width, "update")
+    count = total
+    if rows is not None:
+        _gpu(rows, "rows", torch.int32)
+        count = rows.numel()
+    if weight.shape != (width,) or next_weight.shape != (width,) or out.shape != (count, width):
+        raise KernelError(f"weights must be [{width}] and out [{count}, {width}]")
+    if not (eps > 0.0 and next_eps > 0.0):
+        raise KernelError("eps must be positive")
+    if width > FUSED_NORMS_MAX_WIDTH:
+        if rows is not None:      # the chosen rows alone, and the stream stays as it is: on a copy of those rows
+            picked = h.index_select(0, rows.long())
+            chosen = update.index_select(update.dim() - 2, rows.long())
+            rmsnorm_update(picked, chosen, weight, eps, None)
+            return add_rmsnorm(picked, None, next_weight, next_eps, out)
+        rmsnorm_update(h, update, weight, eps, None)
+        return add_rmsnorm(h, None, next_weight, next_eps, out)
+    _call("stream_ops", "fe_rmsnorm_update_norm", _ptr(h), _ptr(update), c_int(parts), c_longlong(h.numel()), _ptr(weight),
+          c_float(eps), _ptr(next_weight), c_float(next_eps), _ptr(out), c_int(_code(out.dtype)), _ptr(rows),
+          c_int(0 if rows is not None else 1), c_int(count), c_int(width), _stream())
+    return out
+
+
 def rmsnorm_mean(updates, weights: Tensor, eps: float, out: Tensor) -> Tensor:
     """out = mean over b of u_b * rsqrt(mean(u_b^2) + eps) * weights[b]; float32 (an update may
     come as [parts, T, W])."""
@@ -1306,11 +1350,12 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
         raise KernelError("softcap must be positive")
     if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
         raise KernelError("window, chunk and max_q_len must be positive")
-    if (slopes is None and q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
+    if (q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
+            and not (slopes is not None and softcap is not None)
             and block_size >= 16 and block_size & (block_size - 1) == 0 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0):
         paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
                         q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window,
-                        num_decode=num_decode, max_ctx=max_ctx, chunk=chunk, sink=sink, softcap=softcap)
+                        num_decode=num_decode, max_ctx=max_ctx, chunk=chunk, sink=sink, softcap=softcap, slopes=slopes)
         if gate is not None:
             _call("stream_ops", "fe_sigmoid_gate", _ptr(out), _ptr(gate), c_longlong(gate_stride), c_int(_code(out.dtype)),
                   c_int(tokens), c_int(q_heads * value_dim), c_int(value_dim if head_gate else 1), _stream())

@@ -40,7 +40,7 @@ def _mixer(config: MalusunConfig, kind: str, sizes: dict, prefix: str, value_mix
         params["position"] = PartSpec("rotary", {"head_dim": sizes["dim"], "theta": rot["base"], "rotary_dim": rot["dims"],
                                                  "precise": True})
     else:
-        params.update(position=PartSpec("none"), bias=True, output_bias=False, fixed_sink=0.0,
+        params.update(position=PartSpec("none"), bias=True, output_bias=False, bias_init="small", fixed_sink=0.0,
                       distance_slope_bits=DISTANCE_SLOPE_BITS)
     return PartSpec("gqa_attention", params, prefix)
 

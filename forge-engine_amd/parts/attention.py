@@ -55,8 +55,10 @@ class GroupedQueryAttention(Mixer):
                  head_gate: bool = False, whole_norm_eps: float | None = None, softcap: float | None = None,
                  own_kv: bool = True, names: dict[str, str] | None = None, output_bias: bool | None = None,
                  fixed_sink: float | None = None, distance_slope_bits: float | None = None,
-                 value_mix: str | None = None, value_mix_key: str = "values", force_general: bool = False) -> None:
+                 value_mix: str | None = None, value_mix_key: str = "values", force_general: bool = False,
+                 bias_init: str = "zeros") -> None:
         super().__init__(ctx, prefix)
+        self.bias_init = bias_init      # how random models draw the biases of q, k and v ("small": so that they show)
         if num_heads % num_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")
         if head_dim % 2 or not 2 <= head_dim <= 256:
@@ -158,7 +160,7 @@ class GroupedQueryAttention(Mixer):
             if self.own_kv:
                 specs[n["k_norm"]] = ParamSpec((self.kv_size,), kind="vector", init="norm")
         if self.bias:
-            drawn = "small" if self.general else "zeros"      # random models of the general path get biases that show
+            drawn = self.bias_init
             specs[n["q_bias"]] = ParamSpec((self.q_size,), kind="vector", init=drawn)
             specs[n["k_bias"]] = ParamSpec((self.kv_size,), kind="vector", init=drawn)
             specs[n["v_bias"]] = ParamSpec((self.v_size,), kind="vector", init=drawn)

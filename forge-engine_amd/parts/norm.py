@@ -38,8 +38,14 @@ class RMSNorm(Norm):
         self.weight = tensor + self.offset if self.offset else tensor
 
     def forward(self, residual: Residual, rows: Tensor | None = None) -> Tensor:
-        if residual.pending_norm is not None:    # a normed update: into the stream first
-            residual.flush()
+        if residual.pending_norm is not None:    # a norm behind the sublayer before: both norms in one pass over the row
+            if rows is not None:                 # the chosen rows alone; stream and pending update are left as they are
+                update, (weight, eps) = residual.pending, residual.pending_norm
+                out = torch.empty((rows.numel(), self.size), dtype=self.ctx.dtype, device=residual.h.device)
+                return ops.rmsnorm_update_norm(residual.h, update, weight, eps, self.weight, self.eps, out, rows=rows)
+            update, weight, eps = residual.take_normed()
+            out = torch.empty((residual.h.shape[0], self.size), dtype=self.ctx.dtype, device=residual.h.device)
+            return ops.rmsnorm_update_norm(residual.h, update, weight, eps, self.weight, self.eps, out)
         if rows is not None:    # the chosen rows of stream + pending update; both are left as they are
             h = residual.h
             out = torch.empty((rows.numel(), self.size), dtype=self.ctx.dtype, device=h.device)
@@ -49,7 +55,7 @@ class RMSNorm(Norm):
         return ops.add_rmsnorm(residual.h, update, self.weight, self.eps, out)
 
     def kernel_libraries(self):
-        return {"rowwise"}
+        return {"rowwise", "stream_ops"}
 
 
 class UpdateRMSNorm(RMSNorm):

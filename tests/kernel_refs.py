@@ -317,6 +317,17 @@ def rmsnorm_update(h, update, weight, eps, out=None):
     return out
 
 
+def rmsnorm_update_norm(h, update, weight, eps, next_weight, next_eps, out, rows=None):
+    u = _sum_parts(update)
+    v = h + _unit(u, eps) * weight
+    if rows is None:
+        h.copy_(v)
+    else:
+        v = v[rows.long()]
+    out.copy_((_unit(v, next_eps) * next_weight).to(out.dtype))
+    return out
+
+
 def rmsnorm_mean(updates, weights, eps, out):
     total = torch.zeros_like(out)
     for index, update in enumerate(updates):
@@ -695,7 +706,7 @@ NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsno
          "cast_rows", "add_bias", "token_shift", "rmsnorm_update", "rmsnorm_mean", "polynorm", "tanh_rows", "head_norm_gate",
          "conv_rope_norm_write", "masked_attention", "linear_recurrence", "mlstm_gate_scan",
          "hyper_norm", "embed_token_pairs", "scale_rows", "whole_norm_rope_write", "moe_route", "moe_experts", "linear_gated",
-         "relu_squared", "causal_conv_act", "selective_scan")
+         "relu_squared", "causal_conv_act", "selective_scan", "rmsnorm_update_norm")
 
 
 def install(monkeypatch):

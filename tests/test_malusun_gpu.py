@@ -356,3 +356,25 @@ def test_generation_through_the_entry_point_and_the_command_line(folders):
     done = subprocess.run(command, capture_output=True, text=True, timeout=300, env=dict(os.environ))
     assert done.returncode == 0, done.stderr[-2000:]
     assert ",".join(map(str, want[0])) in done.stdout.replace(" ", "")
+
+
+@pytest.mark.parametrize("rows,width,parts", [(1, 40, 1), (37, 256, 3), (9, 2048, 1), (600, 4096, 2), (5, 8192, 1), (3, 9000, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_two_norms_in_one_kernel(rows, width, parts, dtype):
+    """The norm behind a sublayer and the norm before the next: whole steps (the stream moves on) and chosen rows
+    (it does not), updates whole and in parts, rows wider than the fused kernel takes."""
+    from forge_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(rows + width)
+    h = torch.randn(rows, width, generator=g) * 2
+    update = torch.randn(rows, width, generator=g) if parts == 1 else torch.randn(parts, rows, width, generator=g)
+    w, w_next = 1 + 0.2 * torch.randn(width, generator=g), 1 + 0.2 * torch.randn(width, generator=g)
+    pick = torch.tensor([rows - 1, 0, rows - 1], dtype=torch.int32)
+    for chosen in (pick, None):
+        want_h, got_h = h.clone(), h.clone().to(DEV)
+        n = rows if chosen is None else chosen.numel()
+        want = refs.rmsnorm_update_norm(want_h, update, w, 1e-5, w_next, 1e-6, torch.empty(n, width, dtype=dtype), rows=chosen)
+        got = ops.rmsnorm_update_norm(got_h, update.to(DEV), w.to(DEV), 1e-5, w_next.to(DEV), 1e-6,
+                                      torch.empty(n, width, dtype=dtype, device=DEV), rows=None if chosen is None else chosen.to(DEV))
+        close(got, want, dtype)
+        close(got_h, want_h, torch.float32)
+        assert chosen is None or torch.equal(got_h.cpu(), h)
