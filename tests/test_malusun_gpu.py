@@ -75,6 +75,70 @@ def test_convolution_and_selective_scan_kernels(channels, states, taps, dtype):
         close(scan_gpu, scan_ref, torch.float32, loose=5.0)
 
 
+@pytest.mark.parametrize("segment,q_lens", [(16, [70, 1, 0, 33]), (32, [200, 31, 0, 97]), (128, [700, 3, 0, 129]), (64, [64, 128, 0, 65])])
+@pytest.mark.parametrize("channels,states", [(40, 6), (96, 16), (24, 40)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_selective_scan_in_segments(monkeypatch, segment, q_lens, channels, states, dtype):
+    """A step whose sequences are cut into segments that are walked side by side: lengths that end on a
+    segment's edge, one token behind it and one short of it, a sequence inside one segment, an empty one;
+    twice in a row, so that the second step starts from the state the segments' last walk left.  Decays near
+    one, so that a segment's start state matters to its end."""
+    from forge_engine_amd.kernels import ops
+    monkeypatch.setattr(ops, "SCAN_SEGMENT", segment)
+    monkeypatch.setattr(ops, "SCAN_SEGMENT_MIN_TOKENS", 1)
+    g = torch.Generator().manual_seed(channels + states + segment)
+    slots = 5
+    a = -torch.exp(torch.randn(channels, states, generator=g) * 0.5 - 2.0)
+    d, dt_bias = torch.randn(channels, generator=g), torch.randn(channels, generator=g) * 0.5 - 2.0
+    scan_ref = torch.randn(slots, channels, states, generator=g)
+    scan_gpu = scan_ref.clone().to(DEV)
+    for lens in (q_lens, q_lens[::-1]):
+        tokens = sum(lens)
+        assert ops.scan_segment(tokens, 4) == segment
+        cu_q = torch.tensor([sum(lens[:i]) for i in range(5)], dtype=torch.int32)
+        state_slots = torch.tensor([3, 0, 1, 4] if lens is q_lens else [4, slots, 0, 3], dtype=torch.int32)
+        if lens is not q_lens:       # the empty sequence is the second one now
+            assert lens[1] == 0
+        else:
+            state_slots[2] = slots
+        x = torch.randn(tokens, channels, generator=g).to(dtype)
+        z = torch.randn(tokens, channels, generator=g).to(dtype)
+        bc = torch.randn(tokens, 2 * states, generator=g)
+        dt_lin = torch.randn(tokens, channels, generator=g)
+        want = refs.selective_scan(x, dt_lin, dt_bias, a, bc, d, z, scan_ref, cu_q, state_slots, num_seqs=4)
+        got = ops.selective_scan(*to_dev(x, dt_lin, dt_bias, a, bc, d, z), scan_gpu, cu_q.to(DEV), state_slots.to(DEV), num_seqs=4)
+        close(got, want, dtype, loose=5.0)
+        close(scan_gpu, scan_ref, torch.float32, loose=5.0)
+
+
+@pytest.mark.parametrize("taps,q_lens", [(4, [530, 1, 0, 501]), (2, [17, 1000, 0, 15]), (8, [3, 2, 0, 1040]), (1, [600, 400, 0, 48])])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_convolution_over_runs_of_rows(taps, q_lens, dtype):
+    """A step large enough for the convolution's wide shape (four channels a thread, rows in runs that keep
+    the taps' rows in registers): sequences that begin inside a run, at its first and at its last row, so
+    that rows of the state and of another sequence's part of the step lie side by side; twice in a row."""
+    from forge_engine_amd.kernels import ops
+    channels, slots = 1024, 5
+    g = torch.Generator().manual_seed(taps)
+    weight, bias = torch.randn(channels, taps, generator=g) * 0.4, torch.randn(channels, generator=g) * 0.1
+    conv_ref = torch.randn(slots, max(taps - 1, 1), channels, generator=g)
+    conv_gpu = conv_ref.clone().to(DEV)
+    for lens in (q_lens, q_lens[::-1]):
+        tokens = sum(lens)
+        cu_q = torch.tensor([sum(lens[:i]) for i in range(5)], dtype=torch.int32)
+        token_seq = torch.tensor([s for s, n in enumerate(lens) for _ in range(n)], dtype=torch.int32)
+        state_slots = torch.tensor([3, 0, 1, 4], dtype=torch.int32)
+        state_slots[lens.index(0)] = slots
+        xz = torch.randn(tokens, 2 * channels, generator=g).to(dtype)
+        want = refs.causal_conv_act(xz[:, channels:], weight, bias, conv_ref if taps > 1 else None, token_seq, cu_q, state_slots,
+                                    num_seqs=4, act="silu")
+        got = ops.causal_conv_act(xz.to(DEV)[:, channels:], weight.to(DEV), bias.to(DEV), conv_gpu if taps > 1 else None,
+                                  token_seq.to(DEV), cu_q.to(DEV), state_slots.to(DEV), num_seqs=4, act="silu")
+        close(got, want, dtype)
+        if taps > 1:
+            close(conv_gpu, conv_ref, torch.float32)
+
+
 def test_scan_shapes_cover_every_size():
     from forge_engine_amd.kernels import ops
     for states in range(1, 257):
