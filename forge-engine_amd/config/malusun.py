@@ -7,7 +7,7 @@ width (``width``), the norms' epsilon (``norm.eps``), a factor on the embedding
 feed-forward (``mlp``: ``kind`` ``dense`` with ``ff``; ``kind`` ``moe`` with ``router.experts``,
 ``router.top``, ``expert.ff`` and optionally ``shared.ff``; or null for none).  Mixer keys:
 ``mamba1``: ``inner``, ``state``, ``dt_rank``, ``conv``; both attentions: ``heads``, ``kv_heads``,
-``dim``, ``vdim``, ``scale``, ``mask.size`` (the sliding window) and optionally ``v_mix``;
+``dim``, ``vdim``, ``scale``, optionally ``mask.size`` (the sliding window) and ``v_mix``;
 ``attention`` also ``rot.dims`` and ``rot.base``.  Every size and constant of a model comes from
 here; nothing is pinned to one checkpoint.
 """
@@ -49,7 +49,8 @@ def _check_attention(raw: dict, where: str, rotates: bool) -> None:
     dim = read.integer("dim")
     read.integer("vdim")
     read.number("scale")
-    KeyReader(_section(raw, "mask", where)).integer("size")
+    if raw.get("mask") is not None:         # without it every earlier token is seen
+        KeyReader(_section(raw, "mask", where)).integer("size")
     read.boolean("v_mix", False)
     if rotates:
         rot = _section(raw, "rot", where)

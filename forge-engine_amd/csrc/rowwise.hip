@@ -4,10 +4,10 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding
-// out[t, :] = float(table[ids[t], :]).  One block per token.
+// out[t, :] = float(table[ids[t], :]) * scale.  One block per token.
 template <typename TW>
 __global__ void embed_rows_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
-                                  float* __restrict__ out, int hidden, int vocab) {
+                                  float* __restrict__ out, int hidden, int vocab, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   float* dst = out + (size_t)t * hidden;
@@ -16,18 +16,18 @@ __global__ void embed_rows_kernel(const int* __restrict__ ids, const TW* __restr
     return;
   }
   const TW* src = table + (size_t)id * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = load_as_float(src + i);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = load_as_float(src + i) * scale;
 }
 
 extern "C" int fe_embed_rows(const int* ids, const void* table, int table_dtype, float* out,
-                             int tokens, int hidden, int vocab, hipStream_t stream) {
+                             int tokens, int hidden, int vocab, float scale, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
   if (hidden <= 0 || vocab <= 0) return FE_BAD_ARGUMENT;
   const int threads = hidden >= 1024 ? 256 : 64;
   if (table_dtype == FE_F32)
-    embed_rows_kernel<float><<<tokens, threads, 0, stream>>>(ids, (const float*)table, out, hidden, vocab);
+    embed_rows_kernel<float><<<tokens, threads, 0, stream>>>(ids, (const float*)table, out, hidden, vocab, scale);
   else if (table_dtype == FE_BF16)
-    embed_rows_kernel<bf16_t><<<tokens, threads, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab);
+    embed_rows_kernel<bf16_t><<<tokens, threads, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab, scale);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();

@@ -68,8 +68,8 @@ def _call(lib_name: str, fn_name: str, *args) -> None:
 
 # ------------------------------------------------------------------ row-wise
 
-def embed_rows(ids: Tensor, table: Tensor, out: Tensor) -> Tensor:
-    """out[t] = float32(table[ids[t]]); ids int32 [T], table [V, H], out float32 [T, H]."""
+def embed_rows(ids: Tensor, table: Tensor, out: Tensor, scale: float = 1.0) -> Tensor:
+    """out[t] = float32(table[ids[t]]) * scale; ids int32 [T], table [V, H], out float32 [T, H]."""
     _gpu(ids, "ids", torch.int32)
     _gpu(table, "table")
     _gpu(out, "out", torch.float32)
@@ -78,7 +78,7 @@ def embed_rows(ids: Tensor, table: Tensor, out: Tensor) -> Tensor:
     if out.shape != (tokens, hidden):
         raise KernelError(f"out must be [{tokens}, {hidden}], got {tuple(out.shape)}")
     _call("rowwise", "fe_embed_rows", _ptr(ids), _ptr(table), c_int(_code(table.dtype)), _ptr(out),
-          c_int(tokens), c_int(hidden), c_int(vocab), _stream())
+          c_int(tokens), c_int(hidden), c_int(vocab), c_float(scale), _stream())
     return out
 
 

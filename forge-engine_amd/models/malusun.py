@@ -33,7 +33,7 @@ def _mixer(config: MalusunConfig, kind: str, sizes: dict, prefix: str, value_mix
         return PartSpec("selective_scan", {"hidden_size": width, "inner": sizes["inner"], "state": sizes["state"],
                                            "dt_rank": sizes["dt_rank"], "conv_taps": sizes["conv"]}, prefix)
     params = {"hidden_size": width, "num_heads": sizes["heads"], "num_kv_heads": sizes["kv_heads"], "head_dim": sizes["dim"],
-              "value_dim": sizes["vdim"], "scale": sizes["scale"], "window": sizes["mask"]["size"], "value_mix": value_mix,
+              "value_dim": sizes["vdim"], "scale": sizes["scale"], "window": (sizes.get("mask") or {}).get("size"), "value_mix": value_mix,
               "names": ATTENTION_NAMES, "force_general": True}
     if kind == "attention":
         rot = sizes["rot"]

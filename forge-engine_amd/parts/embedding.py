@@ -38,13 +38,11 @@ class TokenEmbedding(Embedding):
 
     def forward(self, batch) -> Residual:
         h = torch.empty((batch.num_tokens, self.hidden_size), dtype=torch.float32, device=self.weight.device)
-        ops.embed_rows(batch.token_ids, self.weight, h)
-        if self.scale != 1.0:
-            ops.scale_rows(h, self.scale)
+        ops.embed_rows(batch.token_ids, self.weight, h, self.scale)
         return Residual(h)
 
     def kernel_libraries(self):
-        return {"rowwise"} | ({"hyper"} if self.scale != 1.0 else set())
+        return {"rowwise"}
 
 
 class TokenPairEmbedding(TokenEmbedding):

@@ -13,8 +13,8 @@ from __future__ import annotations
 import torch
 
 
-def embed_rows(ids, table, out):
-    out.copy_(table[ids.long()].float())
+def embed_rows(ids, table, out, scale=1.0):
+    out.copy_(table[ids.long()].float() * scale)
     return out
 
 

@@ -22,8 +22,10 @@ def attention(heads, kv_heads, dim, vdim, window, rot_dims, *, base=10000.0, sca
 
 
 def attention_2(heads, kv_heads, dim, vdim, window, *, scale=0.3, v_mix=True):
-    return "attention_2", {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale,
-                           "mask": {"size": window}, "v_mix": v_mix}
+    sizes = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "v_mix": v_mix}
+    if window is not None:        # without a mask every earlier token is seen
+        sizes["mask"] = {"size": window}
+    return "attention_2", sizes
 
 
 def dense(ff):
@@ -67,10 +69,11 @@ SMALL_C = config(64, 32, [
     layer(scan(32, 3, 2, 2), None),
     layer(scan(16, 20, 4, 3), dense(40)),
 ])
-# attention alone, nothing mixed, keys as wide as values: no state slot is ever read
+# attention alone, nothing mixed, keys as wide as values: no state slot is ever read; a layer without a window
 SMALL_D = config(70, 24, [
     layer(attention(4, 1, 16, 16, 7, 16, v_mix=False), dense(32)),
     layer(attention_2(2, 2, 6, 6, 4, v_mix=False), None),
+    layer(attention_2(2, 1, 8, 4, None, v_mix=False), dense(16)),
 ])
 # sizes that the matrix-core attention and the grouped products' full tiles take on the GPU
 MEDIUM = config(320, 256, [

@@ -142,7 +142,7 @@ def attention_mixer(h, w, p, sizes, positions, kind: str, shared: dict, cache: d
             k, v = torch.cat([cache["k"], k]), torch.cat([cache["v"], v])
             k_positions = torch.cat([cache["pos"], positions])
         cache["k"], cache["v"], cache["pos"] = k, v, k_positions
-    out = windowed_attention(q, k, v, positions, k_positions, scale=sizes["scale"], window=sizes["mask"]["size"],
+    out = windowed_attention(q, k, v, positions, k_positions, scale=sizes["scale"], window=(sizes.get("mask") or {}).get("size", 1 << 40),
                              slopes=distance_slopes(heads) if kind == "attention_2" else None,
                              one_more=kind == "attention_2")
     return out.reshape(count, heads * vdim) @ w[p + ".o"].T

@@ -36,9 +36,10 @@ def test_embed_rows(ops, dtype, hidden):
     g = torch.Generator().manual_seed(0)
     table = rand(g, 77, hidden, dtype=dtype)
     ids = torch.tensor([0, 76, 5, 5, 31], dtype=torch.int32)
-    want = refs.embed_rows(ids, table, torch.empty(5, hidden))
-    got = ops.embed_rows(ids.to(DEV), table.to(DEV), torch.empty(5, hidden, device=DEV))
-    torch.testing.assert_close(got.cpu(), want, atol=0, rtol=0)
+    for scale in (1.0, 0.75, 3.0):
+        want = refs.embed_rows(ids, table, torch.empty(5, hidden), scale)
+        got = ops.embed_rows(ids.to(DEV), table.to(DEV), torch.empty(5, hidden, device=DEV), scale)
+        torch.testing.assert_close(got.cpu(), want, atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
