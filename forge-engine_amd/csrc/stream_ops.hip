@@ -149,8 +149,9 @@ extern "C" int fe_rmsnorm_update(float* h, const float* update, int parts, long 
 // A norm behind a sublayer and the norm before the next one in one pass over the row:
 //   v = h[s] + u * rsqrt(mean(u^2) + eps) * w        (u = the sum of the update's parts; written back to h if `store`)
 //   out[r] = v * rsqrt(mean(v^2) + eps_next) * w_next,  s = rows[r] or r.
-// The row (up to 8 elements a thread) stays in registers between the three passes.
-template <typename TO>
+// The row (up to 8 elements a thread) stays in registers between the three passes.  VEC 4: a thread's
+// elements are two runs of four neighbours (16-byte loads and stores; the width a multiple of four).
+template <typename TO, int VEC>
 __global__ __launch_bounds__(ROW_THREADS_FEW) void rmsnorm_update_norm_kernel(
     float* __restrict__ h, const float* __restrict__ update, int parts, size_t part_stride,
     const float* __restrict__ w, float eps, const float* __restrict__ w_next, float eps_next, TO* __restrict__ out,
@@ -159,32 +160,71 @@ __global__ __launch_bounds__(ROW_THREADS_FEW) void rmsnorm_update_norm_kernel(
   const size_t base = (size_t)(rows ? rows[blockIdx.x] : (int)blockIdx.x) * width;
   const size_t out_base = (size_t)blockIdx.x * width;
   const int threads = blockDim.x;
+  constexpr int RUNS = 8 / VEC;
   float u[8];
   float ss = 0.f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int c = threadIdx.x + j * threads;
-    u[j] = c < width ? parts_sum(update + base + c, parts, part_stride) : 0.f;
-    ss += u[j] * u[j];
+  for (int j = 0; j < RUNS; ++j) {
+    const int c = (threadIdx.x + j * threads) * VEC;
+    if constexpr (VEC == 4) {
+      float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c < width) {
+        sum = *reinterpret_cast<const float4*>(update + base + c);
+        for (int k = 1; k < parts; ++k) {
+          const float4 more = *reinterpret_cast<const float4*>(update + k * part_stride + base + c);
+          sum.x += more.x; sum.y += more.y; sum.z += more.z; sum.w += more.w;
+        }
+      }
+      u[4 * j] = sum.x; u[4 * j + 1] = sum.y; u[4 * j + 2] = sum.z; u[4 * j + 3] = sum.w;
+      ss += sum.x * sum.x + sum.y * sum.y + sum.z * sum.z + sum.w * sum.w;
+    } else {
+      u[j] = c < width ? parts_sum(update + base + c, parts, part_stride) : 0.f;
+      ss += u[j] * u[j];
+    }
   }
   ss = block_sum<true>(ss, scratch);
   const float inv = rsqrtf(ss / (float)width + eps);
   float ss_next = 0.f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int c = threadIdx.x + j * threads;
+  for (int j = 0; j < RUNS; ++j) {
+    const int c = (threadIdx.x + j * threads) * VEC;
     if (c < width) {
-      u[j] = h[base + c] + u[j] * inv * w[c];
-      if (store) h[base + c] = u[j];
-      ss_next += u[j] * u[j];
+      if constexpr (VEC == 4) {
+        const float4 before = *reinterpret_cast<const float4*>(h + base + c);
+        const float4 weight = *reinterpret_cast<const float4*>(w + c);
+        float4 v;
+        v.x = before.x + u[4 * j] * inv * weight.x;
+        v.y = before.y + u[4 * j + 1] * inv * weight.y;
+        v.z = before.z + u[4 * j + 2] * inv * weight.z;
+        v.w = before.w + u[4 * j + 3] * inv * weight.w;
+        if (store) *reinterpret_cast<float4*>(h + base + c) = v;
+        u[4 * j] = v.x; u[4 * j + 1] = v.y; u[4 * j + 2] = v.z; u[4 * j + 3] = v.w;
+        ss_next += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+      } else {
+        u[j] = h[base + c] + u[j] * inv * w[c];
+        if (store) h[base + c] = u[j];
+        ss_next += u[j] * u[j];
+      }
     }
   }
   ss_next = block_sum(ss_next, scratch);
   const float inv_next = rsqrtf(ss_next / (float)width + eps_next);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int c = threadIdx.x + j * threads;
-    if (c < width) store_from_float(out + out_base + c, u[j] * inv_next * w_next[c]);
+  for (int j = 0; j < RUNS; ++j) {
+    const int c = (threadIdx.x + j * threads) * VEC;
+    if (c < width) {
+      if constexpr (VEC == 4) {
+        const float4 weight = *reinterpret_cast<const float4*>(w_next + c);
+        struct alignas(sizeof(TO) * 4) Pack { TO e[4]; } pack;
+        store_from_float(&pack.e[0], u[4 * j] * inv_next * weight.x);
+        store_from_float(&pack.e[1], u[4 * j + 1] * inv_next * weight.y);
+        store_from_float(&pack.e[2], u[4 * j + 2] * inv_next * weight.z);
+        store_from_float(&pack.e[3], u[4 * j + 3] * inv_next * weight.w);
+        *reinterpret_cast<Pack*>(out + out_base + c) = pack;
+      } else {
+        store_from_float(out + out_base + c, u[j] * inv_next * w_next[c]);
+      }
+    }
   }
 }
 
@@ -196,15 +236,19 @@ extern "C" int fe_rmsnorm_update_norm(float* h, const float* update, int parts, 
   if (count <= 0) return FE_OK;
   const int threads = width > 8 * ROW_THREADS ? ROW_THREADS_FEW : row_threads(count, width);
   if (width <= 0 || width > 8 * threads || parts < 1 || parts > 64 || !(eps > 0.f) || !(eps_next > 0.f) || !out ||
-      (rows && store))
+      (rows && store) || (out_dtype != FE_F32 && out_dtype != FE_BF16))
     return FE_BAD_ARGUMENT;
-  if (out_dtype == FE_F32)
-    rmsnorm_update_norm_kernel<float><<<count, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, w_next,
-                                                                     eps_next, (float*)out, rows, store, width);
-  else if (out_dtype == FE_BF16)
-    rmsnorm_update_norm_kernel<bf16_t><<<count, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, w_next,
-                                                                      eps_next, (bf16_t*)out, rows, store, width);
-  else return FE_BAD_ARGUMENT;
+  const bool wide = width % 4 == 0 && part_stride % 4 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)update % 16 == 0 &&
+                    (uintptr_t)w % 16 == 0 && (uintptr_t)w_next % 16 == 0 && (uintptr_t)out % 16 == 0;
+#define LAUNCH(TO, VEC)                                                                                               \
+  rmsnorm_update_norm_kernel<TO, VEC><<<count, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, w_next, \
+                                                                     eps_next, (TO*)out, rows, store, width)
+  if (out_dtype == FE_F32) {
+    if (wide) LAUNCH(float, 4); else LAUNCH(float, 1);
+  } else {
+    if (wide) LAUNCH(bf16_t, 4); else LAUNCH(bf16_t, 1);
+  }
+#undef LAUNCH
   return fe_check_launch();
 }
 

@@ -422,7 +422,7 @@ def test_generation_through_the_entry_point_and_the_command_line(folders):
     assert ",".join(map(str, want[0])) in done.stdout.replace(" ", "")
 
 
-@pytest.mark.parametrize("rows,width,parts", [(1, 40, 1), (37, 256, 3), (9, 2048, 1), (600, 4096, 2), (5, 8192, 1), (3, 9000, 2)])
+@pytest.mark.parametrize("rows,width,parts", [(1, 40, 1), (37, 256, 3), (9, 2048, 1), (600, 4096, 2), (5, 8192, 1), (3, 9000, 2), (11, 50, 2), (530, 1022, 1), (2100, 2048, 2)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_two_norms_in_one_kernel(rows, width, parts, dtype):
     """The norm behind a sublayer and the norm before the next: whole steps (the stream moves on) and chosen rows
