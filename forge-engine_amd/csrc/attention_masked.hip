@@ -7,7 +7,10 @@
 //   * values of another width than keys;
 //   * an output gate: the result times sigmoid(gate), a gate per element or one per query head;
 //   * a soft cap: scores, after the scale, become cap * tanh(score / cap);
-//   * a penalty on distance: slope_h * (p - j) comes off head h's score of key j (after scale and cap).
+//   * a penalty on distance: slope_h * (p - j) comes off head h's score of key j (after scale and cap);
+//   * a bias by distance: table[h][min(p - j, span - 1)] is added to head h's score of key j (after the scale,
+//     which does not multiply it); the table is float32 [heads][span];
+//   * keys that are their own values (no value pages): a key's first Dv dims are read as its value.
 // One launch serves portions of prompts and single tokens alike; the step's own keys and values are
 // already in the pages (keys [page][kv head][slot][D], values transposed [page][kv head][Dv][slot]).
 // Block = (tile of 16 rows, kv head, sequence), a row being a (query token, head of the group) pair,
@@ -24,14 +27,15 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     T* __restrict__ out, const T* __restrict__ gate, size_t gate_stride, const float* __restrict__ sink,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int D, int Dv, int block_size, int num_blocks, int window,
-    int chunk, float scale, float softcap, int head_gate, const float* __restrict__ slopes) {
+    int chunk, float scale, float softcap, int head_gate, const float* __restrict__ slopes,
+    const float* __restrict__ dist_bias, int span) {
   constexpr int KPT = TK / 16;
   extern __shared__ float smem[];
   const int ks = D + 1, vs = Dv + 1;
   float* Qs = smem;                 // [ROWS][D + 1]
   float* Ks = Qs + ROWS * ks;       // [TK][D + 1]
   float* Vs = Ks + TK * ks;         // [TK][Dv + 1]
-  float* Ps = Vs + TK * vs;         // [ROWS][TK]
+  float* Ps = Vs + (value_pages ? TK * vs : 0);   // [ROWS][TK]; keys that are their own values keep no value tile
 
   const int seq = blockIdx.z, hk = blockIdx.y;
   const int q0 = cu_q[seq];
@@ -73,6 +77,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
 
   const int head = hk * groups + my_g;
   const float slope = slopes ? slopes[head] : 0.f;
+  const float* bias_row = dist_bias ? dist_bias + (size_t)head * span : nullptr;
   float m = sink ? sink[head] : -INFINITY;
   float l = sink ? 1.f : 0.f;
   float acc[DPT];
@@ -93,7 +98,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
       }
       Ks[kk * ks + d] = v;
     }
-    for (int e = tid; e < TK * Dv; e += 256) {
+    for (int e = tid; value_pages && e < TK * Dv; e += 256) {
       const int d = e / TK, kk = e - d * TK;
       const int kp = kt + kk;
       float v = 0.f;
@@ -123,6 +128,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
       float score = s[i] * scale;
       if (softcap > 0.f) score = softcap * tanhf(score / softcap);
       if (slopes) score -= slope * (float)(my_pos - kp);
+      if (bias_row && visible) score += bias_row[min(my_pos - kp, span - 1)];
       s[i] = visible ? score : -INFINITY;
       tile_max = fmaxf(tile_max, s[i]);
     }
@@ -153,7 +159,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     const float* prow = Ps + r * TK;
     for (int kk = 0; kk < TK; ++kk) {
       const float p = prow[kk];
-      const float* vrow = Vs + kk * vs;
+      const float* vrow = value_pages ? Vs + kk * vs : Ks + kk * ks;
 #pragma unroll
       for (int i = 0; i < DPT; ++i)
         if (c + 16 * i < Dv) acc[i] = fmaf(p, vrow[c + 16 * i], acc[i]);
@@ -183,25 +189,36 @@ static int launch_masked(const void* q, long long q_stride, const void* key_page
                          const void* gate, long long gate_stride, const float* sink, const int* cu_q,
                          const int* ctx_len, const int* block_table, int table_stride, int num_seqs, int max_q_len,
                          int q_heads, int kv_heads, int D, int Dv, int block_size, int num_blocks, int window,
-                         int chunk, float scale, float softcap, int head_gate, const float* slopes, hipStream_t stream) {
+                         int chunk, float scale, float softcap, int head_gate, const float* slopes, const float* dist_bias,
+                         int span, hipStream_t stream) {
   const int groups = q_heads / kv_heads;
   const long long rows = (long long)max_q_len * groups;
   const dim3 grid((unsigned)((rows + ROWS - 1) / ROWS), kv_heads, num_seqs);
-  const int tk = D + Dv <= 256 ? 32 : 16;
-  const size_t lds = ((size_t)ROWS * (D + 1) + (size_t)tk * (D + 1) + (size_t)tk * (Dv + 1) + (size_t)ROWS * tk) * sizeof(float);
+  const int held = value_pages ? Dv + 1 : 0;      // values that are the keys' own dims need no tile of their own
+  const int tk = D + held <= 256 ? 32 : 16;
+  const size_t lds = ((size_t)ROWS * (D + 1) + (size_t)tk * (D + 1) + (size_t)tk * held + (size_t)ROWS * tk) * sizeof(float);
 #define LAUNCH(TK, DPT)                                                                                          \
-  masked_attention_kernel<T, TK, DPT><<<grid, 256, lds, stream>>>(                                               \
-      (const T*)q, (size_t)q_stride, (const T*)key_pages, (const T*)value_pages, (T*)out, (const T*)gate,        \
-      (size_t)gate_stride, sink, cu_q, ctx_len, block_table, table_stride, kv_heads, groups, D, Dv, block_size, \
-      num_blocks, window, chunk, scale, softcap, head_gate, slopes)
+  do {                                                                                                           \
+    if (lds > 64 * 1024 &&                                                                                       \
+        hipFuncSetAttribute((const void*)masked_attention_kernel<T, TK, DPT>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)lds) != hipSuccess)                                                             \
+      return FE_BAD_ARGUMENT;                                                                                    \
+    masked_attention_kernel<T, TK, DPT><<<grid, 256, lds, stream>>>(                                             \
+        (const T*)q, (size_t)q_stride, (const T*)key_pages, (const T*)value_pages, (T*)out, (const T*)gate,      \
+        (size_t)gate_stride, sink, cu_q, ctx_len, block_table, table_stride, kv_heads, groups, D, Dv, block_size, \
+        num_blocks, window, chunk, scale, softcap, head_gate, slopes, dist_bias, span);                          \
+  } while (0)
+  if (lds > 150 * 1024) return FE_BAD_ARGUMENT;
   if (tk == 32) {
     if (Dv <= 64) LAUNCH(32, 4);
     else if (Dv <= 128) LAUNCH(32, 8);
-    else LAUNCH(32, 16);
+    else if (Dv <= 256) LAUNCH(32, 16);
+    else LAUNCH(32, 32);
   } else {
     if (Dv <= 64) LAUNCH(16, 4);
     else if (Dv <= 128) LAUNCH(16, 8);
-    else LAUNCH(16, 16);
+    else if (Dv <= 256) LAUNCH(16, 16);
+    else LAUNCH(16, 32);
   }
 #undef LAUNCH
   return fe_check_launch();
@@ -213,10 +230,10 @@ extern "C" int fe_masked_attention(const void* q, int dtype, long long q_stride,
                                    int table_stride, int num_seqs, int max_q_len, int q_heads, int kv_heads,
                                    int head_dim, int value_dim, int block_size, int num_blocks, int window, int chunk,
                                    float scale, float softcap, int head_gate, int tokens, const float* slopes,
-                                   hipStream_t stream) {
+                                   const float* dist_bias, int span, hipStream_t stream) {
   if (tokens <= 0 || num_seqs <= 0) return FE_OK;
-  if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || head_dim < 1 || head_dim > 256 || value_dim < 1 ||
-      value_dim > 256 || block_size <= 0 || num_blocks <= 0 || max_q_len < 1 || window < 0 || chunk < 0 ||
+  if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || head_dim < 1 || head_dim > 640 || value_dim < 1 ||
+      value_dim > 512 || (!value_pages && value_dim > head_dim) || (dist_bias && span < 1) || block_size <= 0 || num_blocks <= 0 || max_q_len < 1 || window < 0 || chunk < 0 ||
       num_seqs > 65535 || kv_heads > 65535)
     return FE_BAD_ARGUMENT;
   if (q_stride < (long long)q_heads * head_dim || softcap < 0.f ||
@@ -225,10 +242,10 @@ extern "C" int fe_masked_attention(const void* q, int dtype, long long q_stride,
   if (dtype == FE_F32)
     return launch_masked<float>(q, q_stride, key_pages, value_pages, out, gate, gate_stride, sink, cu_q, ctx_len,
                                 block_table, table_stride, num_seqs, max_q_len, q_heads, kv_heads, head_dim, value_dim,
-                                block_size, num_blocks, window, chunk, scale, softcap, head_gate, slopes, stream);
+                                block_size, num_blocks, window, chunk, scale, softcap, head_gate, slopes, dist_bias, span, stream);
   if (dtype == FE_BF16)
     return launch_masked<bf16_t>(q, q_stride, key_pages, value_pages, out, gate, gate_stride, sink, cu_q, ctx_len,
                                  block_table, table_stride, num_seqs, max_q_len, q_heads, kv_heads, head_dim, value_dim,
-                                 block_size, num_blocks, window, chunk, scale, softcap, head_gate, slopes, stream);
+                                 block_size, num_blocks, window, chunk, scale, softcap, head_gate, slopes, dist_bias, span, stream);
   return FE_BAD_ARGUMENT;
 }

@@ -9,6 +9,8 @@
 // The projection's bias (float32, one entry per q, k and v channel, or none) is added here, to the
 // rows as they are loaded, so that the product before this kernel has none; the state holds rows
 // with their bias.  One wave per token and head; everything between the loads and the stores is float32.
+// The unit norm may carry a weight per dim, one for q heads and one for k heads, shared by the heads
+// (an RMS norm); with `norm_first` the norm comes before the rotation instead of behind it.
 // Values may lean on another layer's values of the same tokens: v <- (1 - mix) v + mix * v_from
 // (v_from [T, kv_heads * value_dim], dense), after the bias and the convolution and before the page
 // write; a layer that others lean on leaves its values, as stored, in v_keep (same shape).
@@ -26,7 +28,8 @@ __global__ __launch_bounds__(64) void conv_rope_norm_write_kernel(
     const int* __restrict__ state_slots, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ key_pages, T* __restrict__ value_pages, T* __restrict__ q_out, int q_heads, int kv_heads,
     int head_dim, int value_dim, int rotary_dim, float eps, int unit_norm, int taps, int block_size,
-    int num_blocks, int slots, const T* __restrict__ v_from, float v_mix, T* __restrict__ v_keep) {
+    int num_blocks, int slots, const T* __restrict__ v_from, float v_mix, T* __restrict__ v_keep,
+    const float* __restrict__ norm_wq, const float* __restrict__ norm_wk, int norm_first) {
   __shared__ float y[CR_HEAD_MAX];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int seq = token_seq[t];
@@ -76,7 +79,19 @@ __global__ __launch_bounds__(64) void conv_rope_norm_write_kernel(
     return;
   }
 
-  // 2. rotation, a pair per lane
+  // 2. the norm where it comes first; rotation, a pair per lane
+  const float* norm_w = is_q ? norm_wq : norm_wk;
+  auto unit = [&]() {
+    float ss = 0.f;
+    for (int d = lane; d < n; d += 64) ss += y[d] * y[d];
+    ss = wave_sum(ss);
+    return rsqrtf(ss / (float)head_dim + eps);
+  };
+  if (unit_norm && norm_first) {
+    const float inv = unit();
+    for (int d = lane; d < n; d += 64) y[d] = y[d] * inv * (norm_w ? norm_w[d] : 1.f);
+    __syncthreads();
+  }
   const int half = rotary_dim / 2;
   for (int i = lane; i < half; i += 64) {
     float sn, cs;
@@ -87,20 +102,16 @@ __global__ __launch_bounds__(64) void conv_rope_norm_write_kernel(
   }
   __syncthreads();
 
-  // 3. unit norm and the store
+  // 3. the norm behind the rotation, and the store
   float inv = 1.f;
-  if (unit_norm) {
-    float ss = 0.f;
-    for (int d = lane; d < n; d += 64) ss += y[d] * y[d];
-    ss = wave_sum(ss);
-    inv = rsqrtf(ss / (float)head_dim + eps);
-  }
+  const bool late = unit_norm && !norm_first;
+  if (late) inv = unit();
   if (is_q) {
     T* dst = q_out + (size_t)t * q_size + head * head_dim;
-    for (int d = lane; d < n; d += 64) store_from_float(dst + d, y[d] * inv);
+    for (int d = lane; d < n; d += 64) store_from_float(dst + d, y[d] * inv * (late && norm_w ? norm_w[d] : 1.f));
   } else if (paged) {
     T* dst = key_pages + (((size_t)page * kv_heads + (head - q_heads)) * block_size + place) * head_dim;
-    for (int d = lane; d < n; d += 64) store_from_float(dst + d, y[d] * inv);
+    for (int d = lane; d < n; d += 64) store_from_float(dst + d, y[d] * inv * (late && norm_w ? norm_w[d] : 1.f));
   }
 }
 
@@ -137,13 +148,14 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
                                        void* q_out, int tokens, int q_heads, int kv_heads, int head_dim, int value_dim,
                                        int rotary_dim, float eps, int unit_norm, int taps, int block_size,
                                        int num_blocks, int slots, const void* v_from, float v_mix, void* v_keep,
-                                       hipStream_t stream) {
+                                       const float* norm_wq, const float* norm_wk, int norm_first, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
   if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || value_dim <= 0 || block_size <= 0 || num_blocks <= 0)
     return FE_BAD_ARGUMENT;
   if (rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 || (rotary_dim && !inv_freq)) return FE_BAD_ARGUMENT;
   if (taps < 0 || taps > 8 || (taps && !conv_w) || (taps > 1 && (!conv_state || slots < 1))) return FE_BAD_ARGUMENT;
   if (unit_norm && !(eps > 0.f)) return FE_BAD_ARGUMENT;
+  if (!unit_norm && (norm_wq || norm_wk || norm_first)) return FE_BAD_ARGUMENT;
   const long long channels = (long long)(q_heads + kv_heads) * head_dim + (long long)kv_heads * value_dim;
   if (head_dim > CR_HEAD_MAX || value_dim > CR_HEAD_MAX || qkv_stride < channels || q_heads + 2 * kv_heads > 65535)
     return FE_BAD_ARGUMENT;      // a head lives in LDS
@@ -152,7 +164,8 @@ extern "C" int fe_conv_rope_norm_write(const void* qkv, int dtype, long long qkv
   conv_rope_norm_write_kernel<T><<<grid, 64, 0, stream>>>(                                         \
       (const T*)qkv, (size_t)qkv_stride, bias, conv_w, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, \
       block_table, table_stride, (T*)key_pages, (T*)value_pages, (T*)q_out, q_heads, kv_heads, head_dim,       \
-      value_dim, rotary_dim, eps, unit_norm, taps, block_size, num_blocks, slots, (const T*)v_from, v_mix, (T*)v_keep)
+      value_dim, rotary_dim, eps, unit_norm, taps, block_size, num_blocks, slots, (const T*)v_from, v_mix, (T*)v_keep, \
+      norm_wq, norm_wk, norm_first)
   if (dtype == FE_F32) LAUNCH(float);
   else if (dtype == FE_BF16) LAUNCH(bf16_t);
   else return FE_BAD_ARGUMENT;

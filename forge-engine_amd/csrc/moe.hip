@@ -63,6 +63,85 @@ extern "C" int fe_moe_select(const float* logits, const float* bias, int* chosen
   return fe_check_launch();
 }
 
+// Selection by corrected scores within the best groups.  Per token: s = softmax(z) over all E experts; an
+// expert's choice score is s_e + correction_e; the experts form `groups` equal runs of neighbours, a run's score is
+// its largest choice score, and only experts of the `keep` best runs can be chosen (the lowest index among
+// equals, for runs and for experts); the `top` largest choice scores among those are chosen, and their weights are
+// their own s, divided by the sum of the chosen s (+ 1e-20), times `scale`.  The logits' rows lie `stride`
+// floats apart (columns beyond E, a gate's logit say, are not read here).  One thread a token.
+#define SELECT_MAX_GROUPS 64
+__global__ void moe_select_grouped_kernel(const float* __restrict__ z, size_t stride, const float* __restrict__ correction,
+                                          int* __restrict__ chosen, float* __restrict__ weights, int tokens, int E, int top,
+                                          int groups, int keep, float scale) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= tokens) return;
+  const float* row = z + (size_t)t * stride;
+  float peak = -INFINITY;
+  for (int e = 0; e < E; ++e) peak = fmaxf(peak, row[e]);
+  float denom = 0.f;
+  for (int e = 0; e < E; ++e) denom += expf(row[e] - peak);
+  const float inv = 1.f / denom;
+  auto score = [&](int e) { return expf(row[e] - peak) * inv; };
+  auto choice = [&](int e) { return score(e) + (correction ? correction[e] : 0.f); };
+  const int each = E / groups;
+  unsigned long long open = ~0ull;          // bit g: run g may be chosen from
+  if (keep < groups) {
+    float best[SELECT_MAX_GROUPS];
+    for (int g = 0; g < groups; ++g) {
+      float b = -INFINITY;
+      for (int e = g * each; e < (g + 1) * each; ++e) b = fmaxf(b, choice(e));
+      best[g] = b;
+    }
+    open = 0ull;
+    for (int k = 0; k < keep; ++k) {
+      int arg = -1;
+      float value = -INFINITY;
+      for (int g = 0; g < groups; ++g)
+        if (!((open >> g) & 1ull) && (arg < 0 || best[g] > value)) {
+          value = best[g];
+          arg = g;
+        }
+      open |= 1ull << arg;
+    }
+  }
+  int picked[16];
+  float own[16];
+  float total = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int arg = -1;
+    float value = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      if (!((open >> (e / each)) & 1ull)) continue;
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken = taken || picked[j] == e;
+      if (taken) continue;
+      const float v = choice(e);
+      if (arg < 0 || v > value) {
+        value = v;
+        arg = e;
+      }
+    }
+    picked[k] = arg;
+    own[k] = score(arg);
+    total += own[k];
+    chosen[(size_t)t * top + k] = arg;
+  }
+  const float norm = scale / (total + 1e-20f);
+  for (int k = 0; k < top; ++k) weights[(size_t)t * top + k] = own[k] * norm;
+}
+
+extern "C" int fe_moe_select_grouped(const float* logits, long long stride, const float* correction, int* chosen,
+                                     float* weights, int tokens, int experts, int top, int groups, int keep, float scale,
+                                     hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (experts <= 0 || experts > 1024 || top < 1 || top > 16 || stride < experts || groups < 1 ||
+      groups > SELECT_MAX_GROUPS || experts % groups || keep < 1 || keep > groups || top > (experts / groups) * keep)
+    return FE_BAD_ARGUMENT;
+  moe_select_grouped_kernel<<<(tokens + 63) / 64, 64, 0, stream>>>(logits, (size_t)stride, correction, chosen, weights, tokens,
+                                                                   experts, top, groups, keep, scale);
+  return fe_check_launch();
+}
+
 // One block: offsets[e] = pairs of experts below e, order[offsets[e] ..] = the pairs of expert e.
 // Within an expert the pairs come in no fixed order; a pair's results do not depend on its row.
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ chosen, int pairs, int E,

@@ -146,6 +146,81 @@ extern "C" int fe_rmsnorm_update(float* h, const float* update, int parts, long 
   return fe_check_launch();
 }
 
+// h[r] += factor * (u - mean(u)) * rsqrt(var(u) + eps) * w, u = the sum of the update's parts, var the mean
+// of the squared deviations; out (if any) = new h.  A row of up to 8 elements a thread stays in
+// registers between the three passes; wider rows are read again.
+template <typename TO, bool HAS_OUT>
+__global__ __launch_bounds__(ROW_THREADS_FEW) void layernorm_update_kernel(
+    float* __restrict__ h, const float* __restrict__ update, int parts, size_t part_stride,
+    const float* __restrict__ w, float eps, float factor, TO* __restrict__ out, int width) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * width;
+  const int threads = blockDim.x;
+  const bool held = width <= 8 * threads;
+  float u[8];
+  float sum = 0.f;
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = threadIdx.x + j * threads;
+      u[j] = c < width ? parts_sum(update + base + c, parts, part_stride) : 0.f;
+      sum += u[j];
+    }
+  } else {
+    for (int c = threadIdx.x; c < width; c += threads) sum += parts_sum(update + base + c, parts, part_stride);
+  }
+  const float mean = block_sum<true>(sum, scratch) / (float)width;
+  float ss = 0.f;
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = threadIdx.x + j * threads;
+      const float d = c < width ? u[j] - mean : 0.f;
+      ss += d * d;
+    }
+  } else {
+    for (int c = threadIdx.x; c < width; c += threads) {
+      const float d = parts_sum(update + base + c, parts, part_stride) - mean;
+      ss += d * d;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / (float)width + eps) * factor;
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = threadIdx.x + j * threads;
+      if (c < width) {
+        const float v = h[base + c] + (u[j] - mean) * inv * w[c];
+        h[base + c] = v;
+        if (HAS_OUT) store_from_float(out + base + c, v);
+      }
+    }
+  } else {
+    for (int c = threadIdx.x; c < width; c += threads) {
+      const float v = h[base + c] + (parts_sum(update + base + c, parts, part_stride) - mean) * inv * w[c];
+      h[base + c] = v;
+      if (HAS_OUT) store_from_float(out + base + c, v);
+    }
+  }
+}
+
+extern "C" int fe_layernorm_update(float* h, const float* update, int parts, long long part_stride, const float* w,
+                                   float eps, float factor, void* out, int out_dtype, int rows, int width,
+                                   hipStream_t stream) {
+  if (rows <= 0) return FE_OK;
+  if (width <= 0 || parts < 1 || parts > 64 || !(eps > 0.f)) return FE_BAD_ARGUMENT;
+  const int threads = row_threads(rows, width);
+  if (out == nullptr || out_dtype < 0)
+    layernorm_update_kernel<float, false><<<rows, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, factor, nullptr, width);
+  else if (out_dtype == FE_F32)
+    layernorm_update_kernel<float, true><<<rows, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, factor, (float*)out, width);
+  else if (out_dtype == FE_BF16)
+    layernorm_update_kernel<bf16_t, true><<<rows, threads, 0, stream>>>(h, update, parts, (size_t)part_stride, w, eps, factor, (bf16_t*)out, width);
+  else return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
 // A norm behind a sublayer and the norm before the next one in one pass over the row:
 //   v = h[s] + u * rsqrt(mean(u^2) + eps) * w        (u = the sum of the update's parts; written back to h if `store`)
 //   out[r] = v * rsqrt(mean(v^2) + eps_next) * w_next,  s = rows[r] or r.
@@ -407,6 +482,59 @@ extern "C" int fe_relu_squared(const void* x, void* out, int dtype, long long co
   if (dtype == FE_F32) relu_squared_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>((const float*)x, (float*)out, count);
   else if (dtype == FE_BF16) relu_squared_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, count);
   else return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
+// An activation over every element, float32 inside: 0 the square of relu, 1 the gelu with the error
+// function, 0.5 z (1 + erf(z / sqrt 2)), 2 its tanh form, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
+template <typename T, int KIND>
+__global__ void activate_kernel(const T* __restrict__ x, T* __restrict__ out, long long count) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const float z = load_as_float(x + i);
+  float v;
+  if (KIND == 0) {
+    v = fmaxf(z, 0.f);
+    v = v * v;
+  } else if (KIND == 1) {
+    v = 0.5f * z * (1.f + erff(z * 0.70710678118654752440f));
+  } else {
+    v = 0.5f * z * (1.f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+  }
+  store_from_float(out + i, v);
+}
+
+extern "C" int fe_activate(const void* x, void* out, int dtype, long long count, int kind, hipStream_t stream) {
+  if (count <= 0) return FE_OK;
+  const long long blocks = (count + 255) / 256;
+  if (blocks > 0x7fffffffLL || kind < 0 || kind > 2 || (dtype != FE_F32 && dtype != FE_BF16)) return FE_BAD_ARGUMENT;
+#define LAUNCH(T, KIND) activate_kernel<T, KIND><<<(unsigned)blocks, 256, 0, stream>>>((const T*)x, (T*)out, count)
+  if (dtype == FE_F32) {
+    if (kind == 0) LAUNCH(float, 0); else if (kind == 1) LAUNCH(float, 1); else LAUNCH(float, 2);
+  } else {
+    if (kind == 0) LAUNCH(bf16_t, 0); else if (kind == 1) LAUNCH(bf16_t, 1); else LAUNCH(bf16_t, 2);
+  }
+#undef LAUNCH
+  return fe_check_launch();
+}
+
+// update[p][t][c] *= sigmoid(gate[t * gate_stride]): one gate a row, float32, over every part of an update.
+__global__ void gate_rows_kernel(float* __restrict__ update, const float* __restrict__ gate, size_t gate_stride,
+                                 int rows, int width, long long count) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const long long t = (i / width) % rows;
+  update[i] *= 1.f / (1.f + expf(-gate[(size_t)t * gate_stride]));
+}
+
+extern "C" int fe_gate_rows(float* update, int parts, const float* gate, long long gate_stride, int rows, int width,
+                            hipStream_t stream) {
+  if (rows <= 0) return FE_OK;
+  if (width <= 0 || parts < 1 || gate_stride < 1) return FE_BAD_ARGUMENT;
+  const long long count = (long long)parts * rows * width;
+  const long long blocks = (count + 255) / 256;
+  if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  gate_rows_kernel<<<(unsigned)blocks, 256, 0, stream>>>(update, gate, (size_t)gate_stride, rows, width, count);
   return fe_check_launch();
 }
 

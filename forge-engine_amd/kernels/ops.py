@@ -1085,6 +1085,29 @@ def rmsnorm_update(h: Tensor, update: Tensor, weight: Tensor, eps: float, out: T
     return out
 
 
+def layernorm_update(h: Tensor, update: Tensor, weight: Tensor, eps: float, factor: float = 1.0,
+                     out: Tensor | None = None) -> Tensor | None:
+    """h += factor * (u - mean(u)) * rsqrt(var(u) + eps) * weight, u the update (float32, [parts, T, W] added up
+    in order first), var the mean of the squared deviations; all float32.  ``out`` (compute dtype [T, W])
+    receives the new h as well."""
+    _gpu(h, "h", torch.float32)
+    _gpu(weight, "weight", torch.float32)
+    rows, width = h.shape
+    parts = _parts_of(update, rows, width, "update")
+    if weight.shape != (width,):
+        raise KernelError(f"weight must be [{width}]")
+    if out is not None:
+        _gpu(out, "out")
+        if out.shape != h.shape:
+            raise KernelError("out must have the stream's shape")
+    if not eps > 0.0:
+        raise KernelError("eps must be positive")
+    _call("stream_ops", "fe_layernorm_update", _ptr(h), _ptr(update), c_int(parts), c_longlong(h.numel()), _ptr(weight),
+          c_float(eps), c_float(factor), _ptr(out), c_int(_code(out.dtype) if out is not None else -1), c_int(rows),
+          c_int(width), _stream())
+    return out
+
+
 FUSED_NORMS_MAX_WIDTH = 8192       # 8 elements a thread at 1,024 threads a row
 
 
@@ -1221,7 +1244,9 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
                          positions: Tensor, token_seq: Tensor, cu_q: Tensor, state_slots: Tensor, block_table: Tensor,
                          key_pages: Tensor, value_pages: Tensor, q_out: Tensor, *, num_seqs: int, q_heads: int,
                          kv_heads: int, head_dim: int, value_dim: int, rotary_dim: int, unit_norm_eps: float | None,
-                         taps: int, v_from: Tensor | None = None, v_mix: float = 0.0, v_keep: Tensor | None = None) -> None:
+                         taps: int, v_from: Tensor | None = None, v_mix: float = 0.0, v_keep: Tensor | None = None,
+                         norm_weight_q: Tensor | None = None, norm_weight_k: Tensor | None = None,
+                         norm_first: bool = False) -> None:
     """From the projection's output to queries and cached keys and values in one kernel: a short
     projection's bias (float32 [channels] or None: the product before has none), a short causal
     convolution over time on every q, k and v channel (``taps`` > 0: y_t = sum_j c[:, j] *
@@ -1232,8 +1257,17 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
     k and v into their pages (values transposed).  float32 inside, one rounding at the stores.
     qkv [T, >= channels] with any row stride.  ``v_from`` ([T, kv_heads * value_dim], another layer's values of
     the same tokens): the values become ``(1 - v_mix) v + v_mix v_from`` before they are stored; ``v_keep`` (same
-    shape) receives the values as stored, for layers that lean on this one's."""
+    shape) receives the values as stored, for layers that lean on this one's.  ``norm_weight_q`` / ``norm_weight_k``
+    (float32 [head_dim], shared by the heads): the unit norm's result times a weight per dim, an RMS norm;
+    ``norm_first``: the norm comes before the rotation instead of behind it."""
     channels = (q_heads + kv_heads) * head_dim + kv_heads * value_dim
+    for name, w in (("norm_weight_q", norm_weight_q), ("norm_weight_k", norm_weight_k)):
+        if w is not None:
+            _gpu(w, name, torch.float32)
+            if w.shape != (head_dim,) or unit_norm_eps is None:
+                raise KernelError(f"{name} must be [{head_dim}] and comes with a unit norm")
+    if norm_first and unit_norm_eps is None:
+        raise KernelError("norm_first comes with a unit norm")
     _gpu(qkv, "qkv", contiguous=False)
     tokens = qkv.shape[0]
     if qkv.dim() != 2 or qkv.shape[1] < channels or qkv.stride(1) != 1:
@@ -1287,26 +1321,29 @@ def conv_rope_norm_write(qkv: Tensor, bias: Tensor | None, conv_weight: Tensor |
           _ptr(key_pages), _ptr(value_pages), _ptr(q_out), c_int(tokens), c_int(q_heads), c_int(kv_heads), c_int(head_dim),
           c_int(value_dim), c_int(rotary_dim), c_float(unit_norm_eps if unit_norm_eps is not None else 0.0),
           c_int(1 if unit_norm_eps is not None else 0), c_int(taps), c_int(block_size), c_int(num_blocks), c_int(slots),
-          _ptr(v_from), c_float(v_mix), _ptr(v_keep), _stream())
+          _ptr(v_from), c_float(v_mix), _ptr(v_keep), _ptr(norm_weight_q), _ptr(norm_weight_k), c_int(1 if norm_first else 0),
+          _stream())
     if taps > 1:
         _call("conv_rope", "fe_conv_state_update", _ptr(qkv), c_int(_code(qkv.dtype)), c_longlong(stride), _ptr(bias), _ptr(conv_state),
               _ptr(cu_q), _ptr(state_slots), c_int(num_seqs), c_int(channels), c_int(taps), c_int(slots), c_int(tokens),
               _stream())
 
 
-def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor, ctx_len: Tensor,
+def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor | None, out: Tensor, cu_q: Tensor, ctx_len: Tensor,
                      block_table: Tensor, *, num_seqs: int, max_q_len: int, q_heads: int, kv_heads: int, head_dim: int,
                      value_dim: int, scale: float, window: int | None = None, chunk: int | None = None,
                      sink: Tensor | None = None, gate: Tensor | None = None, num_decode: int | None = None,
                      max_ctx: int | None = None, softcap: float | None = None, head_gate: bool = False,
-                     slopes: Tensor | None = None) -> Tensor:
+                     slopes: Tensor | None = None, dist_bias: Tensor | None = None) -> Tensor:
     """Paged grouped-query attention with the masks and softmax forms beyond the causal one: the
     query at position p reads keys j <= p with j > p - window (``window``) and j >= p - p % chunk
     (``chunk``); ``sink`` (float32 [Hq]) adds exp(sink_h) to head h's softmax denominator, with
     no key and no value; values may be of another width than keys; ``gate`` ([T, Hq * Dv] rows of
     any stride; with ``head_gate`` [T, Hq], one number a head) multiplies the result by sigmoid(gate);
     ``softcap``: scores, after the scale, become cap * tanh(score / cap); ``slopes`` (float32 [Hq]): head h's score
-    of key j loses slopes[h] * (p - j).  out [T, Hq * Dv].  Scores and softmax
+    of key j loses slopes[h] * (p - j); ``dist_bias`` (float32 [Hq, span]): head h's score of key j gains
+    dist_bias[h, min(p - j, span - 1)] (after the scale, which does not multiply it); ``value_pages`` None: a key's
+    first ``value_dim`` dims are its value (a cache of keys only).  out [T, Hq * Dv].  Scores and softmax
     float32.  A bfloat16 cache with keys and values of 64 or 128 elements, groups up to 8 and pages of
     a power of two >= 16 goes to the matrix-core kernels of ``paged_attention`` (single tokens and
     portions each to its own), with the gate in a small kernel behind them; everything else, and
@@ -1314,7 +1351,8 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
     _gpu(q, "q", contiguous=False)
     _gpu(out, "out", q.dtype)
     _gpu(key_pages, "key_pages", q.dtype)
-    _gpu(value_pages, "value_pages", q.dtype)
+    if value_pages is not None:
+        _gpu(value_pages, "value_pages", q.dtype)
     _gpu(cu_q, "cu_q", torch.int32)
     _gpu(ctx_len, "ctx_len", torch.int32)
     _gpu(block_table, "block_table", torch.int32)
@@ -1322,12 +1360,14 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
     q_stride = _strided_rows(q, "q", q_heads * head_dim)
     if out.shape != (tokens, q_heads * value_dim):
         raise KernelError(f"out must be [{tokens}, {q_heads * value_dim}], got {tuple(out.shape)}")
-    if q_heads % kv_heads or not 1 <= head_dim <= 256 or not 1 <= value_dim <= 256:
-        raise KernelError("query heads must be a multiple of kv heads, head sizes in [1, 256]")
+    if q_heads % kv_heads or not 1 <= head_dim <= MASKED_MAX_KEY_DIM or not 1 <= value_dim <= MASKED_MAX_VALUE_DIM:
+        raise KernelError(f"query heads must be a multiple of kv heads, keys of up to {MASKED_MAX_KEY_DIM} and values of up to {MASKED_MAX_VALUE_DIM} dims")
+    if value_pages is None and value_dim > head_dim:
+        raise KernelError("values that are the keys' own dims cannot be wider than the keys")
     if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
         raise KernelError(f"key pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
     num_blocks, _, block_size, _ = key_pages.shape
-    if value_pages.shape != (num_blocks, kv_heads, value_dim, block_size):
+    if value_pages is not None and value_pages.shape != (num_blocks, kv_heads, value_dim, block_size):
         raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {value_dim}, block_size]")
     if cu_q.numel() != num_seqs + 1 or ctx_len.numel() != num_seqs or block_table.shape[0] < num_seqs:
         raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
@@ -1341,6 +1381,12 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
         _gpu(slopes, "slopes", torch.float32)
         if slopes.shape != (q_heads,):
             raise KernelError(f"slopes must be [{q_heads}]")
+    span = 0
+    if dist_bias is not None:
+        _gpu(dist_bias, "dist_bias", torch.float32)
+        if dist_bias.dim() != 2 or dist_bias.shape[0] != q_heads or dist_bias.shape[1] < 1:
+            raise KernelError(f"dist_bias must be [{q_heads}, span >= 1], got {tuple(dist_bias.shape)}")
+        span = dist_bias.shape[1]
     gate_stride = 0
     if gate is not None:
         gate_stride = _strided_rows(gate, "gate", q_heads if head_gate else q_heads * value_dim)
@@ -1351,7 +1397,7 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
     if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
         raise KernelError("window, chunk and max_q_len must be positive")
     if (q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
-            and not (slopes is not None and softcap is not None)
+            and not (slopes is not None and softcap is not None) and dist_bias is None and value_pages is not None
             and block_size >= 16 and block_size & (block_size - 1) == 0 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0):
         paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
                         q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window,
@@ -1365,8 +1411,109 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Ten
           _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(q_heads),
           c_int(kv_heads), c_int(head_dim), c_int(value_dim), c_int(block_size), c_int(num_blocks),
           c_int(window or 0), c_int(chunk or 0), c_float(scale), c_float(softcap or 0.0), c_int(1 if head_gate else 0),
-          c_int(tokens), _ptr(slopes), _stream())
+          c_int(tokens), _ptr(slopes), _ptr(dist_bias), c_int(span), _stream())
     return out
+
+
+MASKED_MAX_KEY_DIM = 640        # what the vector-ALU attention kernel holds of a key tile in LDS
+MASKED_MAX_VALUE_DIM = 512
+
+
+# ------------------------------------------------- attention through a latent
+
+def latent_norm_rope_write(x: Tensor, q_weight: Tensor, kv_weight: Tensor | None, inv_freq: Tensor | None, positions: Tensor,
+                           token_seq: Tensor, block_table: Tensor | None, key_pages: Tensor | None, cq_out: Tensor, *, q_rank: int,
+                           kv_rank: int, rot_dim: int, rotary_dim: int, eps: float, write_kv: bool) -> Tensor:
+    """From a token's fused down-projections x = [a | b | r] (float32 [T, >= q_rank (+ kv_rank + rot_dim)], any
+    row stride): ``cq_out`` [T, q_rank] = a / rms(a) * q_weight, and with ``write_kv`` the token's cache row
+    [b / rms(b) * kv_weight | rotate(r)] into ``key_pages`` [blocks, 1, block_size, kv_rank + rot_dim] (a cache of
+    keys only).  The rotation turns the first ``rotary_dim`` dims of r, dim i with dim i + rotary_dim / 2, by
+    position * inv_freq[i].  Norms and angles float32 (epsilon inside the root), one rounding at the stores."""
+    _gpu(x, "x", torch.float32, contiguous=False)
+    _gpu(q_weight, "q_weight", torch.float32)
+    _gpu(cq_out, "cq_out")
+    tokens = x.shape[0]
+    need = q_rank + (kv_rank + rot_dim if write_kv else 0)
+    if x.dim() != 2 or x.shape[1] < need or (x.shape[1] > 1 and x.stride(1) != 1):
+        raise KernelError(f"x must be [T, >= {need}] with unit inner stride, got {tuple(x.shape)}")
+    if q_weight.shape != (q_rank,) or cq_out.shape != (tokens, q_rank) or not eps > 0.0:
+        raise KernelError(f"q_weight must be [{q_rank}], cq_out [{tokens}, {q_rank}] and eps positive")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= rot_dim:
+        raise KernelError("rotary_dim must be even and at most rot_dim")
+    block_size = num_blocks = table_stride = 0
+    if write_kv:
+        _gpu(kv_weight, "kv_weight", torch.float32)
+        _gpu(key_pages, "key_pages", cq_out.dtype)
+        _gpu(block_table, "block_table", torch.int32)
+        _gpu(positions, "positions", torch.int32)
+        _gpu(token_seq, "token_seq", torch.int32)
+        if kv_weight.shape != (kv_rank,) or positions.numel() != tokens or token_seq.numel() != tokens:
+            raise KernelError(f"kv_weight must be [{kv_rank}], positions and token_seq hold one entry per token")
+        if key_pages.dim() != 4 or key_pages.shape[1] != 1 or key_pages.shape[3] != kv_rank + rot_dim:
+            raise KernelError(f"key pages must be [blocks, 1, block_size, {kv_rank + rot_dim}], got {tuple(key_pages.shape)}")
+        if block_table.dim() != 2 or block_table.stride(1) != 1:
+            raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
+        if rotary_dim:
+            _gpu(inv_freq, "inv_freq", torch.float32)
+            if inv_freq.shape != (rotary_dim // 2,):
+                raise KernelError(f"inv_freq must be [{rotary_dim // 2}]")
+        num_blocks, _, block_size, _ = key_pages.shape
+        table_stride = block_table.stride(0)
+    stride = x.stride(0) if tokens > 1 else max(x.stride(0), x.shape[1])
+    _call("latent", "fe_latent_norm_rope_write", _ptr(x), c_longlong(stride), c_int(q_rank), c_int(kv_rank), c_int(rot_dim),
+          c_int(rotary_dim), _ptr(q_weight), _ptr(kv_weight if write_kv else None), _ptr(inv_freq if write_kv and rotary_dim else None),
+          _ptr(positions if write_kv else None), _ptr(token_seq if write_kv else None), _ptr(block_table if write_kv else None),
+          c_int(table_stride), _ptr(key_pages if write_kv else None), _ptr(cq_out), c_int(_code(cq_out.dtype)), c_float(eps),
+          c_int(tokens), c_int(block_size), c_int(num_blocks), c_int(1 if write_kv else 0), _stream())
+    return cq_out
+
+
+def latent_query_pack(q: Tensor, qa: Tensor, inv_freq: Tensor | None, positions: Tensor, out: Tensor, *, heads: int, dim: int,
+                      rot_dim: int, rotary_dim: int, kv_rank: int) -> Tensor:
+    """The attention's query rows ``out`` [T, heads, kv_rank + rot_dim]: head h's first kv_rank dims are
+    ``qa[h, t]`` (qa [heads, T, kv_rank]: the queries taken through the keys' up-projection), the rest the
+    last rot_dim dims of head h of ``q`` [T, heads * (dim + rot_dim)], their first ``rotary_dim`` rotated
+    (dim i with dim i + rotary_dim / 2, angle position * inv_freq[i], float32)."""
+    _gpu(q, "q", contiguous=False)
+    _gpu(qa, "qa", q.dtype)
+    _gpu(out, "out", q.dtype)
+    _gpu(positions, "positions", torch.int32)
+    tokens = q.shape[0]
+    q_stride = _strided_rows(q, "q", heads * (dim + rot_dim))
+    if qa.shape != (heads, tokens, kv_rank) or out.shape != (tokens, heads, kv_rank + rot_dim) or positions.numel() != tokens:
+        raise KernelError(f"qa must be [{heads}, {tokens}, {kv_rank}] and out [{tokens}, {heads}, {kv_rank + rot_dim}]")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= rot_dim:
+        raise KernelError("rotary_dim must be even and at most rot_dim")
+    if rotary_dim:
+        _gpu(inv_freq, "inv_freq", torch.float32)
+        if inv_freq.shape != (rotary_dim // 2,):
+            raise KernelError(f"inv_freq must be [{rotary_dim // 2}]")
+    _call("latent", "fe_latent_query_pack", _ptr(q), c_longlong(q_stride), _ptr(qa), _ptr(inv_freq if rotary_dim else None),
+          _ptr(positions), _ptr(out), c_int(_code(q.dtype)), c_int(tokens), c_int(heads), c_int(dim), c_int(rot_dim),
+          c_int(rotary_dim), c_int(kv_rank), _stream())
+    return out
+
+
+def latent_attention(q: Tensor, key_pages: Tensor, out: Tensor, cu_q: Tensor, ctx_len: Tensor, block_table: Tensor, *,
+                     num_seqs: int, max_q_len: int, heads: int, row_dim: int, value_dim: int, scale: float,
+                     num_decode: int | None = None, max_ctx: int | None = None) -> Tensor:
+    """Causal attention of ``heads`` query heads over one shared cache of keys only, ``key_pages`` [blocks, 1,
+    block_size, row_dim]: a row is the key of every head and its first ``value_dim`` dims are the value.  q
+    [T, heads * row_dim], out [T, heads * value_dim]; scores and softmax float32."""
+    return masked_attention(q, key_pages, None, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
+                            q_heads=heads, kv_heads=1, head_dim=row_dim, value_dim=value_dim, scale=scale,
+                            num_decode=num_decode, max_ctx=max_ctx)
+
+
+def heads_product(x: Tensor, weight: Tensor) -> Tensor:
+    """A product per head: x [T, heads, K] (rows and heads of any stride, unit inner stride) times weight
+    [heads, K, N] gives [heads, T, N] in x's dtype, accumulated in float32 (true float32 products for
+    float32 operands).  The platform's batched matrix product."""
+    _gpu(x, "x", contiguous=False)
+    _gpu(weight, "weight", x.dtype, contiguous=False)
+    if x.dim() != 3 or weight.dim() != 3 or weight.shape[0] != x.shape[1] or weight.shape[1] != x.shape[2]:
+        raise KernelError(f"x must be [T, heads, K] and weight [heads, K, N], got {tuple(x.shape)} and {tuple(weight.shape)}")
+    return torch.bmm(x.transpose(0, 1), weight)
 
 
 # ------------------------------------------------- linear recurrences over a matrix state
@@ -1620,6 +1767,36 @@ def moe_route(x: Tensor, router_weight: Tensor, router_bias: Tensor | None, top:
     return chosen, weights
 
 
+def moe_route_grouped(x: Tensor, router_weight: Tensor, correction: Tensor | None, *, experts: int, top: int, groups: int = 1,
+                      keep: int = 1, scale: float = 1.0) -> tuple[Tensor, Tensor, Tensor]:
+    """Router logits ``x W^T`` in float32 (W may hold rows beyond the ``experts`` first, a gate's say: their logits
+    come back with the others); scores s = softmax over the experts' logits; an expert's choice score is
+    ``s + correction``; the experts form ``groups`` equal runs of neighbours, a run's score is its largest
+    choice score, and only experts of the ``keep`` best runs can be chosen; the ``top`` largest choice scores
+    are chosen (int32 [T, top], largest first, the lowest index among equals) and their weights (float32
+    [T, top]) are their own s over the sum of the chosen s (+ 1e-20), times ``scale``.  Returns (chosen,
+    weights, logits [T, rows of W])."""
+    _gpu(x, "x")
+    _gpu(router_weight, "router_weight", x.dtype)
+    tokens, hidden = x.shape
+    if router_weight.dim() != 2 or router_weight.shape[1] != hidden or router_weight.shape[0] < experts:
+        raise KernelError(f"router_weight must be [>= {experts}, {hidden}], got {tuple(router_weight.shape)}")
+    if not 1 <= experts <= 1024 or not 1 <= groups <= 64 or experts % groups or not 1 <= keep <= groups:
+        raise KernelError("up to 1,024 experts in up to 64 equal groups, of which between one and all are kept")
+    if not 1 <= top <= min(16, experts // groups * keep):
+        raise KernelError(f"top must lie between 1 and min(16, experts of the kept groups), got {top}")
+    if correction is not None:
+        _gpu(correction, "correction", torch.float32)
+        if correction.shape != (experts,):
+            raise KernelError(f"correction must be [{experts}]")
+    logits = linear(x, router_weight, out_dtype=torch.float32)
+    chosen = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
+    _call("moe", "fe_moe_select_grouped", _ptr(logits), c_longlong(logits.shape[1]), _ptr(correction), _ptr(chosen), _ptr(weights),
+          c_int(tokens), c_int(experts), c_int(top), c_int(groups), c_int(keep), c_float(scale), _stream())
+    return chosen, weights, logits
+
+
 def moe_experts(x: Tensor, chosen: Tensor, weights: Tensor, gate_up: Tensor, down: Tensor, out: Tensor, *, limit: float = 0.0,
                 alpha: float = 1.0, extra: Tensor | None = None, form: str = "bounded", weight_input: bool = False) -> Tensor:
     """out[k, t] = weights[t, k] * down[e] @ act, e = chosen[t, k], with ``act = min(g, limit) *
@@ -1685,6 +1862,34 @@ def relu_squared(x: Tensor) -> Tensor:
     out = torch.empty_like(x)
     _call("stream_ops", "fe_relu_squared", _ptr(x), _ptr(out), c_int(_code(x.dtype)), c_longlong(x.numel()), _stream())
     return out
+
+
+ACTIVATIONS = {"relu_squared": 0, "gelu": 1, "gelu_tanh": 2}
+
+
+def activate(x: Tensor, kind: str) -> Tensor:
+    """An activation of every element, into a new tensor of x's dtype (float32 inside): ``relu_squared``,
+    ``gelu`` (0.5 z (1 + erf(z / sqrt 2))) or ``gelu_tanh`` (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))))."""
+    _gpu(x, "x")
+    if kind not in ACTIVATIONS:
+        raise KernelError(f"unknown activation '{kind}' (known: {', '.join(ACTIVATIONS)})")
+    out = torch.empty_like(x)
+    _call("stream_ops", "fe_activate", _ptr(x), _ptr(out), c_int(_code(x.dtype)), c_longlong(x.numel()), c_int(ACTIVATIONS[kind]),
+          _stream())
+    return out
+
+
+def gate_rows(update: Tensor, logits: Tensor, column: int) -> Tensor:
+    """update[..., t, :] *= sigmoid(logits[t, column]), in place: one gate a token over a float32 update
+    [T, W] or [parts, T, W]; logits float32 [T, n]."""
+    _gpu(update, "update", torch.float32)
+    _gpu(logits, "logits", torch.float32)
+    if update.dim() not in (2, 3) or logits.dim() != 2 or logits.shape[0] != update.shape[-2] or not 0 <= column < logits.shape[1]:
+        raise KernelError(f"update must be [T, W] or [parts, T, W] and logits [T, > {column}], got {tuple(update.shape)} and {tuple(logits.shape)}")
+    parts = update.shape[0] if update.dim() == 3 else 1
+    _call("stream_ops", "fe_gate_rows", _ptr(update), c_int(parts), c_void_p(logits.data_ptr() + 4 * column), c_longlong(logits.shape[1]),
+          c_int(update.shape[-2]), c_int(update.shape[-1]), _stream())
+    return update
 
 
 def causal_conv_act(u: Tensor, weight: Tensor, bias: Tensor | None, state: Tensor | None, token_seq: Tensor, cu_q: Tensor,

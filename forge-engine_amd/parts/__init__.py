@@ -1,7 +1,7 @@
 """The parts a decoder is assembled from; importing this package registers the
 built-in kinds."""
 
-from . import attention, block, embedding, mlp, moe, norm, parallel, recurrent, rotary, selective_scan  # noqa: F401
+from . import attention, block, embedding, latent_attention, mlp, moe, norm, parallel, recurrent, rotary, selective_scan  # noqa: F401
 from .base import (Block, BuildContext, Embedding, FeedForward, Head, Mixer, Norm, ParamSpec, Part,
                    PositionEncoding, Residual, build_part)
 from .plan import LayerCall, LayerSpec, ModelPlan, PartSpec

@@ -28,6 +28,12 @@ score without key or value: 0 puts a one into the denominator); ``distance_slope
 score of key j loses ``2^(-c (h + 1) / H) * (i - j)``, H heads, after the scale); ``value_mix``
 ("source": the layer leaves its values of the step's tokens for later layers; "blend": its values
 become ``(1 - m) v + m v_source`` with m a scalar tensor of the layer, before they are cached);
+``distance_bias`` (``{"rows": B, "reach": D}``: a learned table [B, H] whose row ``bucket(i - j)`` is
+added to head h's score of key j after the scale, which does not multiply it; ``bucket(n) = n`` below
+B / 2, else ``min(B - 1, B / 2 + floor(ln(n / (B / 2)) / ln(D / (B / 2)) * (B - B / 2)))``: one row a distance
+at first, logarithmic steps beyond, the last row from distance D on; the rows are laid out by distance
+once, when the table is loaded); ``qk_norm_eps`` on the general path (the weighted RMS norm of every q
+and k head, before the rotation, in the kernel that writes the pages);
 ``force_general`` (take the general path whatever the options).  A position part may scale its
 cosines and sines (``magnitude``).  With any of them the step takes the general path:
 one product for q, k, v (and the gate), one kernel for convolution, rotation, norms and the
@@ -56,7 +62,7 @@ class GroupedQueryAttention(Mixer):
                  own_kv: bool = True, names: dict[str, str] | None = None, output_bias: bool | None = None,
                  fixed_sink: float | None = None, distance_slope_bits: float | None = None,
                  value_mix: str | None = None, value_mix_key: str = "values", force_general: bool = False,
-                 bias_init: str = "zeros") -> None:
+                 bias_init: str = "zeros", distance_bias: dict | None = None) -> None:
         super().__init__(ctx, prefix)
         self.bias_init = bias_init      # how random models draw the biases of q, k and v ("small": so that they show)
         if num_heads % num_kv_heads:
@@ -92,6 +98,13 @@ class GroupedQueryAttention(Mixer):
         if self.output_bias and not bias:
             raise ValueError("a bias on the output projection comes with biases on q, k and v")
         self.value_mix, self.value_mix_key = value_mix, value_mix_key
+        self.distance_bias = None
+        if distance_bias is not None:
+            rows, reach = int(distance_bias["rows"]), float(distance_bias["reach"])
+            if rows < 2 or not reach > rows // 2:
+                raise ValueError(f"a table of biases by distance needs two rows or more and a reach beyond half its rows, not {rows} and {reach}")
+            self.distance_bias = (rows, reach)
+        self.bias_table: Tensor | None = None       # as loaded [rows, heads]; by distance [heads, span] after finalize
         self.mix_weight: float | None = None
         self.slopes: Tensor | None = None
         if whole_norm_eps is not None and (self.conv_taps or unit_norm_eps is not None or bias):
@@ -107,11 +120,13 @@ class GroupedQueryAttention(Mixer):
                             or chunk is not None or sink or self.output_gate or whole_norm_eps is not None
                             or softcap is not None or not own_kv or fixed_sink is not None
                             or distance_slope_bits is not None or value_mix is not None
-                            or self.output_bias != bool(bias) or force_general)
+                            or self.output_bias != bool(bias) or force_general or distance_bias is not None)
         if (value_mix is not None or fixed_sink is not None or distance_slope_bits is not None) and whole_norm_eps is not None:
             raise ValueError("value mixing, fixed sinks and distance slopes are not combined with the whole-projection norm")
-        if self.general and qk_norm_eps is not None:
-            raise ValueError("weighted q/k norms before the rotation are not combined with the general path's options")
+        if self.general and qk_norm_eps is not None and (whole_norm_eps is not None or unit_norm_eps is not None):
+            raise ValueError("weighted q/k norms before the rotation are not combined with another norm of q and k")
+        if distance_bias is not None and whole_norm_eps is not None:
+            raise ValueError("biases by distance are not combined with the whole-projection norm")
         self.names = dict(self.DEFAULT_NAMES, **(names or {}))
         self.qk_norm_eps = qk_norm_eps
         self.bias = bias
@@ -143,7 +158,7 @@ class GroupedQueryAttention(Mixer):
         "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
         "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
         "q_conv": "q_proj.conv", "k_conv": "k_proj.conv", "v_conv": "v_proj.conv",
-        "sink": "sink", "gate": "gate_proj.weight", "value_mix": "value_mix",
+        "sink": "sink", "gate": "gate_proj.weight", "value_mix": "value_mix", "distance_bias": "distance_bias",
     }
 
     def param_specs(self):
@@ -175,6 +190,8 @@ class GroupedQueryAttention(Mixer):
             specs[n["v_conv"]] = ParamSpec((self.v_size, self.conv_taps), kind="vector", init="taps")
         if self.sink:
             specs[n["sink"]] = ParamSpec((self.num_heads,), kind="vector", init="unit")
+        if self.distance_bias is not None:
+            specs[n["distance_bias"]] = ParamSpec((self.distance_bias[0], self.num_heads), kind="vector", init="unit")
         if self.output_gate:
             specs[n["gate"]] = ParamSpec((self.gate_size, self.hidden_size))
         if self.value_mix is not None:      # a scalar; the source layer's is never read
@@ -213,6 +230,8 @@ class GroupedQueryAttention(Mixer):
             self.k_norm = tensor
         elif key == "sink":
             self.sink_weight = tensor
+        elif key == "distance_bias" and self.distance_bias is not None:
+            self.bias_table = tensor
         elif key == "value_mix" and self.value_mix is not None:
             self.mix_weight = float(tensor.reshape(()).item())
         else:
@@ -225,6 +244,8 @@ class GroupedQueryAttention(Mixer):
         if self.distance_slope_bits is not None:
             slopes = [2.0 ** (-self.distance_slope_bits * (head + 1) / self.num_heads) for head in range(self.num_heads)]
             self.slopes = torch.tensor(slopes, dtype=torch.float64).to(torch.float32).to(device)
+        if self.distance_bias is not None:
+            self.bias_table = self._bias_by_distance(self.bias_table).to(device)
         # the general path adds biases in float32 behind the products, which then take the kernels for few rows
         self.conv_bias = None if self.qkv_bias is None else self.qkv_bias[:self.conv_channels].float().contiguous()
         self.o_bias_f32 = None if self.o_bias is None else self.o_bias.float().contiguous()
@@ -232,6 +253,25 @@ class GroupedQueryAttention(Mixer):
             self.qkv_bias = self.qkv_bias.to(self.qkv_weight.dtype)
         if self.o_bias is not None and self.o_weight.dtype != torch.float32:
             self.o_bias = self.o_bias.to(self.o_weight.dtype)
+
+    def _bias_by_distance(self, table: Tensor) -> Tensor:
+        """The loaded table [rows, heads] laid out by distance, float32 [heads, span]: entry n is the row of
+        distance n's bucket; the last entry serves every distance from span - 1 on (with a window, no
+        distance beyond window - 1 is ever read; without one, all distances from the reach on share the
+        last row)."""
+        import math
+
+        rows, reach = self.distance_bias
+        half = rows // 2
+        last = int(math.ceil(reach)) if self.window is None else min(self.window - 1, int(math.ceil(reach)))
+        buckets = []
+        for n in range(last + 1):
+            if n < half:
+                buckets.append(n)
+            else:
+                buckets.append(min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(reach / half) * (rows - half)))))
+        index = torch.tensor(buckets, dtype=torch.long, device=table.device)
+        return table.to(torch.float32).index_select(0, index).t().contiguous()
 
     def split_qkv_weight(self) -> dict[str, Tensor]:
         """The three projection matrices back out of the fused one."""
@@ -312,7 +352,7 @@ class GroupedQueryAttention(Mixer):
             q, cache.key_pages, cache.value_pages, attn, batch.cu_q, batch.ctx_len, cache.block_table,
             num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim, scale=self.scale,
-            window=self.window, chunk=self.chunk, sink=self.sink_weight, slopes=self.slopes,
+            window=self.window, chunk=self.chunk, sink=self.sink_weight, slopes=self.slopes, dist_bias=self.bias_table,
             gate=qkv[:, self.conv_channels:] if self.output_gate else None, num_decode=batch.num_decode,
             max_ctx=batch.max_ctx, softcap=self.softcap, head_gate=self.head_gate)
         update = ops.linear_update(attn, self.o_weight)
@@ -333,7 +373,10 @@ class GroupedQueryAttention(Mixer):
             batch.positions, batch.token_seq, batch.cu_q, batch.state_slots, cache.block_table,
             cache.key_pages, cache.value_pages, q, num_seqs=batch.num_seqs, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, value_dim=self.value_dim,
-            rotary_dim=rotary_dim, unit_norm_eps=self.unit_norm_eps, taps=self.conv_taps, **mixing)
+            rotary_dim=rotary_dim, unit_norm_eps=self.unit_norm_eps if self.qk_norm_eps is None else self.qk_norm_eps,
+            taps=self.conv_taps, norm_weight_q=self.q_norm if self.qk_norm_eps is not None else None,
+            norm_weight_k=self.k_norm if self.qk_norm_eps is not None else None,
+            norm_first=self.qk_norm_eps is not None, **mixing)
 
     def _single_tokens_only(self, batch, x: Tensor, cache: CacheView, rotary_dim: int) -> bool:
         """Every sequence of the step brings one token, and the sizes are ones that the

@@ -99,9 +99,10 @@ class PolyNormMLP(FeedForward):
 
 class ActivatedMLP(FeedForward):
     """``down(act(up(x)))`` without a gate and without biases; ``activation``: ``relu_squared``
-    (``max(z, 0)^2``)."""
+    (``max(z, 0)^2``), ``gelu`` (``0.5 z (1 + erf(z / sqrt 2))``) or ``gelu_tanh``
+    (``0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))``)."""
 
-    ACTIVATIONS = ("relu_squared",)
+    ACTIVATIONS = ("relu_squared", "gelu", "gelu_tanh")
 
     def __init__(self, ctx: BuildContext, prefix: str, *, hidden_size: int, intermediate_size: int,
                  activation: str = "relu_squared", names: dict[str, str] | None = None) -> None:
@@ -129,7 +130,8 @@ class ActivatedMLP(FeedForward):
             raise KeyError(name)
 
     def forward(self, x: Tensor, batch=None) -> Tensor:
-        act = ops.relu_squared(ops.linear(x, self.up_weight))
+        z = ops.linear(x, self.up_weight)
+        act = ops.relu_squared(z) if self.activation == "relu_squared" else ops.activate(z, self.activation)
         return ops.linear_update(act, self.down_weight)
 
     def kernel_libraries(self):

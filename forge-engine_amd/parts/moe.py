@@ -11,7 +11,13 @@ Options: ``scoring`` "sigmoid" (a chosen expert's weight is the sigmoid of its o
 renormalised over the chosen); ``form`` "silu" (``y = W_down (silu(W_gate x) * (W_up x))``, no
 bounds); ``weight_input`` (the weight multiplies the expert's input, ``expert(w x)``, instead of
 its output; since the first products are linear, they are scaled behind their sums);
-``router_bias`` False (the router has no bias tensor).
+``router_bias`` False (the router has no bias tensor); ``scoring`` "softmax_all" (scores are the
+softmax over all experts' logits; experts are chosen by score plus a stored ``correction`` per
+expert, within the ``keep_groups`` best of ``groups`` equal runs of neighbouring experts, a run
+being as good as its best corrected score; a chosen expert's weight is its own score over the
+sum of the chosen scores, times ``route_scale``); ``shared_gate`` (the shared expert's output times
+``sigmoid(w_g . x)``, one number a token, w_g a tensor of one row; its logit is formed with the
+router's, in float32).
 
 A step sorts its (token, choice) pairs by expert on the device and runs two grouped products over
 the sorted rows (gate and up with the activation as their ending, then down, weighted by the
@@ -34,7 +40,8 @@ class RoutedExperts(FeedForward):
     def __init__(self, ctx: BuildContext, prefix: str, *, hidden_size: int, experts: int, top: int,
                  intermediate_size: int, limit: float | None = None, alpha: float = 1.702, shared_size: int | None = None,
                  shared_limit: float | None = None, names: dict[str, str] | None = None, scoring: str = "softmax",
-                 form: str = "bounded", weight_input: bool = False, router_bias: bool = True) -> None:
+                 form: str = "bounded", weight_input: bool = False, router_bias: bool = True, groups: int = 1,
+                 keep_groups: int = 1, route_scale: float = 1.0, shared_gate: bool = False) -> None:
         """``names``: what the tensors are called behind the prefix; ``expert`` is a pattern with
         ``{e}`` for the expert's number."""
         super().__init__(ctx, prefix)
@@ -45,8 +52,18 @@ class RoutedExperts(FeedForward):
         self.hidden_size = hidden_size
         self.experts, self.top = experts, top
         self.intermediate_size = intermediate_size
-        if scoring not in ("softmax", "sigmoid") or form not in ("bounded", "silu"):
+        if scoring not in ("softmax", "sigmoid", "softmax_all") or form not in ("bounded", "silu"):
             raise ValueError(f"unknown scoring '{scoring}' or form '{form}'")
+        if scoring == "softmax_all":
+            if not 1 <= groups <= 64 or experts % groups or not 1 <= keep_groups <= groups or top > experts // groups * keep_groups:
+                raise ValueError(f"{experts} experts do not form {groups} equal groups of which {keep_groups} hold {top} choices")
+            if router_bias or weight_input:
+                raise ValueError("scores over all experts come without a router bias and weigh the experts' outputs")
+        elif groups != 1 or keep_groups != 1 or route_scale != 1.0:
+            raise ValueError("groups and a factor on the weights come with scoring 'softmax_all'")
+        if shared_gate and not shared_size:
+            raise ValueError("a gate on the shared expert needs a shared expert")
+        self.groups, self.keep_groups, self.route_scale, self.shared_gate = int(groups), int(keep_groups), float(route_scale), bool(shared_gate)
         if form == "bounded" and limit is None:
             raise ValueError("the bounded activation needs a limit")
         self.scoring, self.form, self.weight_input, self.has_router_bias = scoring, form, bool(weight_input), bool(router_bias)
@@ -54,7 +71,10 @@ class RoutedExperts(FeedForward):
         self.shared_size = shared_size
         self.shared_limit = float(self.limit if shared_limit is None else shared_limit)
         self.names = dict({"expert": "experts.{e}", "shared": "shared", "router": "router.weight", "router_bias": "router.bias",
-                           "gate": "gate", "up": "up", "down": "down"}, **(names or {}))
+                           "gate": "gate", "up": "up", "down": "down", "correction": "correction", "shared_gate": "shared.gate_proj"},
+                          **(names or {}))
+        self.correction: Tensor | None = None
+        self.router_rows: Tensor | None = None      # with a gate on the shared expert: the router's rows, then the gate's row
         self.router_weight: Tensor | None = None
         self.router_bias: Tensor | None = None
         self.gate_up: Tensor | None = None          # [experts, 2 F, H]: an expert's gate rows, then its up rows
@@ -69,6 +89,10 @@ class RoutedExperts(FeedForward):
     def param_specs(self):
         f, h = self.intermediate_size, self.hidden_size
         specs = {self.name(self.names["router"]): ParamSpec((self.experts, h), init="router")}
+        if self.scoring == "softmax_all":     # a checkpoint without it: no correction
+            specs[self.name(self.names["correction"])] = ParamSpec((self.experts,), kind="vector", init="small", optional=True)
+        if self.shared_gate:
+            specs[self.name(self.names["shared_gate"])] = ParamSpec((1, h), init="router")
         if self.has_router_bias:
             specs[self.name(self.names["router_bias"])] = ParamSpec((self.experts,), kind="vector", init="small")
         for expert in range(self.experts):
@@ -87,8 +111,22 @@ class RoutedExperts(FeedForward):
 
     def set_param(self, name: str, tensor: Tensor) -> None:
         f, h = self.intermediate_size, self.hidden_size
-        if name == self.name(self.names["router"]):
-            self.router_weight = tensor.contiguous()
+        if name == self.name(self.names["router"]) or (self.shared_gate and name == self.name(self.names["shared_gate"])):
+            if not self.shared_gate:
+                self.router_weight = tensor.contiguous()
+                return
+            if self.router_rows is None:
+                self.router_rows = torch.empty((self.experts + 1, h), dtype=tensor.dtype, device=tensor.device)
+                self.router_weight = self.router_rows[:self.experts]
+            if tensor.dtype != self.router_rows.dtype:
+                raise ValueError(f"{name}: the router and the shared expert's gate must be stored in one dtype")
+            if name == self.name(self.names["router"]):
+                self.router_rows[:self.experts].copy_(tensor)
+            else:
+                self.router_rows[self.experts:].copy_(tensor)
+            return
+        if self.scoring == "softmax_all" and name == self.name(self.names["correction"]):
+            self.correction = tensor.contiguous()
             return
         if self.has_router_bias and name == self.name(self.names["router_bias"]):
             self.router_bias = tensor.contiguous()
@@ -123,7 +161,16 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x: Tensor, batch=None) -> Tensor:
         tokens = x.shape[0]
-        chosen, weights = ops.moe_route(x, self.router_weight, self.router_bias, self.top, self.scoring)
+        gate_logits, gate_column = None, 0
+        if self.scoring == "softmax_all":
+            chosen, weights, logits = ops.moe_route_grouped(
+                x, self.router_rows if self.shared_gate else self.router_weight, self.correction, experts=self.experts,
+                top=self.top, groups=self.groups, keep=self.keep_groups, scale=self.route_scale)
+            gate_logits, gate_column = logits, self.experts
+        else:
+            chosen, weights = ops.moe_route(x, self.router_weight, self.router_bias, self.top, self.scoring)
+            if self.shared_gate:
+                gate_logits = ops.linear(x, self.router_rows[self.experts:], out_dtype=torch.float32)
         shared = None
         if self.shared_size:
             if self.form == "silu":     # the gated SiLU of the dense feed-forward, with its fused kernels
@@ -131,12 +178,14 @@ class RoutedExperts(FeedForward):
             else:
                 act = ops.linear_gated(x, self.shared_gate_up, limit=self.shared_limit, alpha=self.alpha)
             shared = ops.linear_update(act, self.shared_down)
+            if self.shared_gate:
+                ops.gate_rows(shared, gate_logits, gate_column)
         update = torch.empty((self.top, tokens, self.hidden_size), dtype=torch.float32, device=x.device)
         return ops.moe_experts(x, chosen, weights, self.gate_up, self.down, update, limit=self.limit, alpha=self.alpha,
                                extra=shared, form=self.form, weight_input=self.weight_input)
 
     def kernel_libraries(self):
-        return {"moe", "rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "gemm_tile"}
+        return {"moe", "rowwise", "stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "gemm_tile"}
 
 
 register_part("feed_forward", "routed_experts", RoutedExperts)

@@ -87,8 +87,9 @@ class LayerNorm(Norm):
     reads_streams = True
 
     def __init__(self, ctx: BuildContext, prefix: str, *, size: int, eps: float, leaf: str = "weight",
-                 bias_leaf: str = "bias") -> None:
-        """``leaf`` / ``bias_leaf``: the tensors' names behind the prefix ("": the prefix itself)."""
+                 bias_leaf: str | None = "bias") -> None:
+        """``leaf`` / ``bias_leaf``: the tensors' names behind the prefix ("": the prefix itself);
+        ``bias_leaf`` None: a layer norm with a weight and no bias."""
         super().__init__(ctx, prefix)
         self.size = size
         self.eps = float(eps)
@@ -97,13 +98,15 @@ class LayerNorm(Norm):
         self.bias: Tensor | None = None
 
     def param_specs(self):
-        return {self.name(self.leaf): ParamSpec((self.size,), kind="vector", init="norm"),
-                self.name(self.bias_leaf): ParamSpec((self.size,), kind="vector", init="small")}
+        specs = {self.name(self.leaf): ParamSpec((self.size,), kind="vector", init="norm")}
+        if self.bias_leaf is not None:
+            specs[self.name(self.bias_leaf)] = ParamSpec((self.size,), kind="vector", init="small")
+        return specs
 
     def set_param(self, name: str, tensor: Tensor) -> None:
         if name == self.name(self.leaf):
             self.weight = tensor
-        elif name == self.name(self.bias_leaf):
+        elif self.bias_leaf is not None and name == self.name(self.bias_leaf):
             self.bias = tensor
         else:
             raise KeyError(name)
@@ -122,6 +125,42 @@ class LayerNorm(Norm):
         return {"hyper"}
 
 
+class UpdateLayerNorm(Norm):
+    """Layer norm (a weight, no bias) of a sublayer's output instead of its input: the pending update u
+    becomes ``factor * (u - mean(u)) * rsqrt(var(u) + eps) * w`` (var: the mean of the squared deviations)
+    and is added into the stream, all in float32 and in one kernel.  Returns the new stream in the compute
+    dtype, which is what the next sublayer of such a layer reads."""
+
+    def __init__(self, ctx: BuildContext, prefix: str, *, size: int, eps: float, leaf: str = "weight", factor: float = 1.0) -> None:
+        super().__init__(ctx, prefix)
+        self.size = size
+        self.eps = float(eps)
+        self.leaf = leaf
+        self.factor = float(factor)
+        self.weight: Tensor | None = None
+
+    def param_specs(self):
+        return {self.name(self.leaf): ParamSpec((self.size,), kind="vector", init="norm")}
+
+    def set_param(self, name: str, tensor: Tensor) -> None:
+        if name != self.name(self.leaf):
+            raise KeyError(name)
+        self.weight = tensor
+
+    def forward(self, residual: Residual, rows: Tensor | None = None) -> Tensor:
+        if rows is not None:
+            raise ValueError("a norm of updates serves whole steps, not chosen rows")
+        update, residual.pending = residual.pending, None
+        if update is None:
+            raise ValueError("a norm of updates needs a pending update")
+        out = torch.empty((residual.h.shape[0], self.size), dtype=self.ctx.dtype, device=residual.h.device)
+        return ops.layernorm_update(residual.h, update, self.weight, self.eps, self.factor, out)
+
+    def kernel_libraries(self):
+        return {"stream_ops"}
+
+
 register_part("norm", "layer_norm", LayerNorm)
+register_part("norm", "layer_norm_of_update", UpdateLayerNorm)
 register_part("norm", "rms_norm", RMSNorm)
 register_part("norm", "rms_norm_of_update", UpdateRMSNorm)

@@ -74,4 +74,4 @@ def _load_builtin() -> None:
         return
     _BUILTIN_LOADED = True
     from . import parts  # noqa: F401  registers the built-in parts
-    from .models import malusun, mazanex, qwen3, rekezen  # noqa: F401  register Malusun, Mazanex, Qwen3ForCausalLM and Rekezen
+    from .models import dubizen, malusun, mazanex, qwen3, rekezen  # noqa: F401  register Dubizen, Malusun, Mazanex, Qwen3ForCausalLM and Rekezen

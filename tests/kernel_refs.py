@@ -381,7 +381,8 @@ def add_bias(update, bias):
 
 def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions, token_seq, cu_q, state_slots, block_table,
                          key_pages, value_pages, q_out, *, num_seqs, q_heads, kv_heads, head_dim, value_dim, rotary_dim,
-                         unit_norm_eps, taps, v_from=None, v_mix=0.0, v_keep=None):
+                         unit_norm_eps, taps, v_from=None, v_mix=0.0, v_keep=None, norm_weight_q=None, norm_weight_k=None,
+                         norm_first=False):
     tokens = qkv.shape[0]
     q_size, k_size, v_size = q_heads * head_dim, kv_heads * head_dim, kv_heads * value_dim
     channels = q_size + k_size + v_size
@@ -402,19 +403,21 @@ def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions
             y[a:b] = sum(history[j:j + b - a] * conv_weight[:, j] for j in range(taps))
             conv_state[slot] = history[-(taps - 1):]
 
-    def rotate_norm(x):
+    def rotate_norm(x, weight):
+        if unit_norm_eps is not None and norm_first:
+            x = _unit(x, unit_norm_eps) * (1.0 if weight is None else weight)
         if rotary_dim:
             half = rotary_dim // 2
             angle = positions.float().view(-1, 1, 1) * inv_freq.view(1, 1, half)
             cos, sin = angle.cos(), angle.sin()
             lo, hi = x[..., :half], x[..., half:rotary_dim]
             x = torch.cat((lo * cos - hi * sin, hi * cos + lo * sin, x[..., rotary_dim:]), dim=-1)
-        if unit_norm_eps is not None:
-            x = _unit(x, unit_norm_eps)
+        if unit_norm_eps is not None and not norm_first:
+            x = _unit(x, unit_norm_eps) * (1.0 if weight is None else weight)
         return x
 
-    q = rotate_norm(y[:, :q_size].view(tokens, q_heads, head_dim))
-    k = rotate_norm(y[:, q_size:q_size + k_size].view(tokens, kv_heads, head_dim)).to(qkv.dtype)
+    q = rotate_norm(y[:, :q_size].view(tokens, q_heads, head_dim), norm_weight_q)
+    k = rotate_norm(y[:, q_size:q_size + k_size].view(tokens, kv_heads, head_dim), norm_weight_k).to(qkv.dtype)
     v = y[:, q_size + k_size:]
     if v_from is not None:
         v = (1.0 - v_mix) * v + v_mix * v_from.float()
@@ -433,7 +436,7 @@ def conv_rope_norm_write(qkv, bias, conv_weight, conv_state, inv_freq, positions
 
 def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, q_heads, kv_heads,
                      head_dim, value_dim, scale, window=None, chunk=None, sink=None, gate=None, num_decode=None, max_ctx=None,
-                     softcap=None, head_gate=False, slopes=None):
+                     softcap=None, head_gate=False, slopes=None, dist_bias=None):
     block_size = key_pages.shape[2]
     groups = q_heads // kv_heads
     for s in range(num_seqs):
@@ -442,7 +445,10 @@ def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table,
         if b == a:
             continue
         keys = gather_pages(key_pages, block_table[s], ctx, block_size)                         # [kv, ctx, D]
-        values = gather_pages(value_pages.transpose(2, 3), block_table[s], ctx, block_size)     # [kv, ctx, Dv]
+        if value_pages is None:      # a cache of keys only: a key's first dims are its value
+            values = keys[..., :value_dim]
+        else:
+            values = gather_pages(value_pages.transpose(2, 3), block_table[s], ctx, block_size)     # [kv, ctx, Dv]
         for i in range(b - a):
             p = ctx - (b - a) + i
             first = 0
@@ -458,6 +464,9 @@ def masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table,
                     scores = softcap * torch.tanh(scores / softcap)
                 if slopes is not None:
                     scores = scores - slopes[h] * (p - torch.arange(first, p + 1, device=scores.device)).float()
+                if dist_bias is not None:
+                    distance = (p - torch.arange(first, p + 1, device=scores.device)).clamp(max=dist_bias.shape[1] - 1)
+                    scores = scores + dist_bias[h, distance]
                 top = scores.max()
                 if sink is not None:
                     top = torch.maximum(top, sink[h])
@@ -688,6 +697,106 @@ def selective_scan(x, dt_lin, dt_bias, a, bc, d, z, state, cu_q, state_slots, *,
     return out
 
 
+def layernorm_update(h, update, weight, eps, factor=1.0, out=None):
+    u = _sum_parts(update)
+    centred = u - u.mean(-1, keepdim=True)
+    h += factor * centred * torch.rsqrt(centred.square().mean(-1, keepdim=True) + eps) * weight
+    if out is not None:
+        out.copy_(h.to(out.dtype))
+    return out
+
+
+def activate(x, kind):
+    z = x.float()
+    if kind == "relu_squared":
+        y = torch.relu(z).square()
+    elif kind == "gelu":
+        y = 0.5 * z * (1.0 + torch.erf(z * 0.7071067811865476))
+    elif kind == "gelu_tanh":
+        y = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+    else:
+        raise ValueError(kind)
+    return y.to(x.dtype)
+
+
+def gate_rows(update, logits, column):
+    update *= torch.sigmoid(logits[:, column]).view(-1, 1)
+    return update
+
+
+def _turn(r, positions, inv_freq, rotary_dim):
+    """r [T, ..., n]: its first rotary_dim dims rotated, dim i with dim i + rotary_dim / 2."""
+    if not rotary_dim:
+        return r
+    half = rotary_dim // 2
+    angle = positions.float().view(-1, *([1] * (r.dim() - 2)), 1) * inv_freq.view(*([1] * (r.dim() - 1)), half)
+    cos, sin = angle.cos(), angle.sin()
+    lo, hi = r[..., :half], r[..., half:rotary_dim]
+    return torch.cat((lo * cos - hi * sin, hi * cos + lo * sin, r[..., rotary_dim:]), dim=-1)
+
+
+def latent_norm_rope_write(x, q_weight, kv_weight, inv_freq, positions, token_seq, block_table, key_pages, cq_out, *, q_rank,
+                           kv_rank, rot_dim, rotary_dim, eps, write_kv):
+    x = x.float()
+    cq_out.copy_((_unit(x[:, :q_rank], eps) * q_weight).to(cq_out.dtype))
+    if not write_kv:
+        return cq_out
+    latent = _unit(x[:, q_rank:q_rank + kv_rank], eps) * kv_weight
+    turned = _turn(x[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim], positions, inv_freq, rotary_dim)
+    rows = torch.cat((latent, turned), dim=-1).to(key_pages.dtype)
+    block_size = key_pages.shape[2]
+    for t in range(x.shape[0]):
+        pos = int(positions[t])
+        page = int(block_table[int(token_seq[t]), pos // block_size])
+        assert page >= 0, "token without a page"
+        key_pages[page, 0, pos % block_size] = rows[t]
+    return cq_out
+
+
+def latent_query_pack(q, qa, inv_freq, positions, out, *, heads, dim, rot_dim, rotary_dim, kv_rank):
+    tokens = q.shape[0]
+    turned = _turn(q.view(tokens, heads, dim + rot_dim)[:, :, dim:].float(), positions, inv_freq, rotary_dim)
+    out[:, :, :kv_rank] = qa.transpose(0, 1)
+    out[:, :, kv_rank:] = turned.to(out.dtype)
+    return out
+
+
+def latent_attention(q, key_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, heads, row_dim, value_dim, scale,
+                     num_decode=None, max_ctx=None):
+    block_size = key_pages.shape[2]
+    for s in range(num_seqs):
+        a, b = int(cu_q[s]), int(cu_q[s + 1])
+        ctx = int(ctx_len[s])
+        if b == a:
+            continue
+        rows = gather_pages(key_pages, block_table[s], ctx, block_size)[0]            # [ctx, row_dim]
+        for i in range(b - a):
+            p = ctx - (b - a) + i
+            queries = q[a + i].float().view(heads, row_dim)
+            weights = torch.softmax(queries @ rows[:p + 1].T * scale, dim=-1)         # [heads, p + 1]
+            out[a + i] = (weights @ rows[:p + 1, :value_dim]).reshape(-1).to(out.dtype)
+    return out
+
+
+def heads_product(x, weight):
+    return torch.einsum("thk,hkn->htn", x.float(), weight.float()).to(x.dtype)
+
+
+def moe_route_grouped(x, router_weight, correction, *, experts, top, groups=1, keep=1, scale=1.0):
+    logits = x.float() @ router_weight.float().T
+    scores = torch.softmax(logits[:, :experts], dim=-1)
+    choice = scores if correction is None else scores + correction
+    if keep < groups:
+        best = choice.view(-1, groups, experts // groups).max(-1).values                         # [T, groups]
+        order = torch.argsort(best, dim=-1, descending=True, stable=True)[:, :keep]
+        kept = torch.zeros_like(best, dtype=torch.bool).scatter_(1, order, True)
+        choice = choice.masked_fill(~kept.repeat_interleave(experts // groups, dim=1), float("-inf"))
+    chosen = torch.argsort(choice, dim=-1, descending=True, stable=True)[:, :top]
+    own = scores.gather(1, chosen)
+    weights = own / (own.sum(-1, keepdim=True) + 1e-20) * scale
+    return chosen.to(torch.int32), weights, logits
+
+
 def decode_prepare_supported(*args, **kwargs):
     return False        # on the CPU a step of single tokens takes the two references below in turn
 
@@ -706,7 +815,8 @@ NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsno
          "cast_rows", "add_bias", "token_shift", "rmsnorm_update", "rmsnorm_mean", "polynorm", "tanh_rows", "head_norm_gate",
          "conv_rope_norm_write", "masked_attention", "linear_recurrence", "mlstm_gate_scan",
          "hyper_norm", "embed_token_pairs", "scale_rows", "whole_norm_rope_write", "moe_route", "moe_experts", "linear_gated",
-         "relu_squared", "causal_conv_act", "selective_scan", "rmsnorm_update_norm")
+         "relu_squared", "causal_conv_act", "selective_scan", "rmsnorm_update_norm", "layernorm_update", "activate", "gate_rows",
+         "latent_norm_rope_write", "latent_query_pack", "latent_attention", "heads_product", "moe_route_grouped")
 
 
 def install(monkeypatch):
