@@ -3,7 +3,9 @@
 //   fe_latent_norm_rope_write: from the fused down-projections of a token, x = [a | b | r] (float32: a of
 //       q_rank, b of kv_rank, r of rot_dim entries), the query latent a / rms(a) * wq into cq [T, q_rank] and,
 //       for a layer that caches, the token's cache row [b / rms(b) * wkv | rotate(r)] into its page
-//       (keys only: [page][1][slot][kv_rank + rot_dim]).  The rotation turns the first rotary_dim dims
+//       (key pages [page][1][slot][kv_rank + rot_dim]) and, where the cache keeps values, the normed b a
+//       second time into the transposed value pages ([page][1][kv_rank][slot], the layout the matrix-core
+//       attention reads its second operand in).  The rotation turns the first rotary_dim dims
 //       of r, dim i with dim i + rotary_dim / 2, by the angle position * inv_freq[i]; the rest pass.
 //   fe_latent_query_pack: the attention's query rows [T, heads, kv_rank + rot_dim] from the queries taken
 //       through the key up-projection (qa [heads, T, kv_rank], the result of a batched product) and
@@ -18,8 +20,8 @@ __global__ __launch_bounds__(LT_THREADS) void latent_norm_rope_write_kernel(
     const float* __restrict__ x, size_t stride, int q_rank, int kv_rank, int rot_dim, int rotary_dim,
     const float* __restrict__ wq, const float* __restrict__ wkv, const float* __restrict__ inv_freq,
     const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ block_table,
-    int table_stride, T* __restrict__ key_pages, T* __restrict__ cq, float eps, int block_size, int num_blocks,
-    int write_kv) {
+    int table_stride, T* __restrict__ key_pages, T* __restrict__ value_pages, T* __restrict__ cq, float eps,
+    int block_size, int num_blocks, int write_kv) {
   __shared__ float scratch[16];
   const int t = blockIdx.x, tid = threadIdx.x;
   const float* row = x + (size_t)t * stride;
@@ -39,7 +41,12 @@ __global__ __launch_bounds__(LT_THREADS) void latent_norm_rope_write_kernel(
   const int page = block_table[(size_t)token_seq[t] * table_stride + pos / block_size];
   if (page < 0 || page >= num_blocks) return;
   T* dst = key_pages + ((size_t)page * block_size + pos % block_size) * (kv_rank + rot_dim);
-  for (int c = tid; c < kv_rank; c += LT_THREADS) store_from_float(dst + c, b[c] * inv_b * wkv[c]);
+  T* vdst = value_pages ? value_pages + (size_t)page * kv_rank * block_size + pos % block_size : nullptr;
+  for (int c = tid; c < kv_rank; c += LT_THREADS) {
+    const float v = b[c] * inv_b * wkv[c];
+    store_from_float(dst + c, v);
+    if (vdst) store_from_float(vdst + (size_t)c * block_size, v);
+  }
   const float* r = b + kv_rank;
   const int half = rotary_dim / 2;
   for (int i = tid; i < half; i += LT_THREADS) {
@@ -55,7 +62,7 @@ __global__ __launch_bounds__(LT_THREADS) void latent_norm_rope_write_kernel(
 extern "C" int fe_latent_norm_rope_write(const float* x, long long stride, int q_rank, int kv_rank, int rot_dim,
                                          int rotary_dim, const float* wq, const float* wkv, const float* inv_freq,
                                          const int* positions, const int* token_seq, const int* block_table,
-                                         int table_stride, void* key_pages, void* cq, int dtype, float eps, int tokens,
+                                         int table_stride, void* key_pages, void* value_pages, void* cq, int dtype, float eps, int tokens,
                                          int block_size, int num_blocks, int write_kv, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
   if (q_rank < 1 || kv_rank < 1 || rot_dim < 0 || rotary_dim < 0 || rotary_dim > rot_dim || rotary_dim % 2 || !(eps > 0.f) ||
@@ -68,7 +75,7 @@ extern "C" int fe_latent_norm_rope_write(const float* x, long long stride, int q
 #define LAUNCH(T)                                                                                                 \
   latent_norm_rope_write_kernel<T><<<tokens, LT_THREADS, 0, stream>>>(                                            \
       x, (size_t)stride, q_rank, kv_rank, rot_dim, rotary_dim, wq, wkv, inv_freq, positions, token_seq, block_table, \
-      table_stride, (T*)key_pages, (T*)cq, eps, block_size, num_blocks, write_kv)
+      table_stride, (T*)key_pages, (T*)value_pages, (T*)cq, eps, block_size, num_blocks, write_kv)
   if (dtype == FE_F32) LAUNCH(float);
   else if (dtype == FE_BF16) LAUNCH(bf16_t);
   else return FE_BAD_ARGUMENT;

@@ -1422,12 +1422,14 @@ MASKED_MAX_VALUE_DIM = 512
 # ------------------------------------------------- attention through a latent
 
 def latent_norm_rope_write(x: Tensor, q_weight: Tensor, kv_weight: Tensor | None, inv_freq: Tensor | None, positions: Tensor,
-                           token_seq: Tensor, block_table: Tensor | None, key_pages: Tensor | None, cq_out: Tensor, *, q_rank: int,
-                           kv_rank: int, rot_dim: int, rotary_dim: int, eps: float, write_kv: bool) -> Tensor:
+                           token_seq: Tensor, block_table: Tensor | None, key_pages: Tensor | None, value_pages: Tensor | None,
+                           cq_out: Tensor, *, q_rank: int, kv_rank: int, rot_dim: int, rotary_dim: int, eps: float,
+                           write_kv: bool) -> Tensor:
     """From a token's fused down-projections x = [a | b | r] (float32 [T, >= q_rank (+ kv_rank + rot_dim)], any
     row stride): ``cq_out`` [T, q_rank] = a / rms(a) * q_weight, and with ``write_kv`` the token's cache row
-    [b / rms(b) * kv_weight | rotate(r)] into ``key_pages`` [blocks, 1, block_size, kv_rank + rot_dim] (a cache of
-    keys only).  The rotation turns the first ``rotary_dim`` dims of r, dim i with dim i + rotary_dim / 2, by
+    [b / rms(b) * kv_weight | rotate(r)] into ``key_pages`` [blocks, 1, block_size, kv_rank + rot_dim] and, if the
+    cache keeps values (``value_pages`` [blocks, 1, kv_rank, block_size], transposed), its first kv_rank numbers
+    there as well.  The rotation turns the first ``rotary_dim`` dims of r, dim i with dim i + rotary_dim / 2, by
     position * inv_freq[i].  Norms and angles float32 (epsilon inside the root), one rounding at the stores."""
     _gpu(x, "x", torch.float32, contiguous=False)
     _gpu(q_weight, "q_weight", torch.float32)
@@ -1459,11 +1461,16 @@ def latent_norm_rope_write(x: Tensor, q_weight: Tensor, kv_weight: Tensor | None
                 raise KernelError(f"inv_freq must be [{rotary_dim // 2}]")
         num_blocks, _, block_size, _ = key_pages.shape
         table_stride = block_table.stride(0)
+        if value_pages is not None:
+            _gpu(value_pages, "value_pages", cq_out.dtype)
+            if value_pages.shape != (num_blocks, 1, kv_rank, block_size):
+                raise KernelError(f"value pages are transposed: [blocks, 1, {kv_rank}, block_size], got {tuple(value_pages.shape)}")
     stride = x.stride(0) if tokens > 1 else max(x.stride(0), x.shape[1])
     _call("latent", "fe_latent_norm_rope_write", _ptr(x), c_longlong(stride), c_int(q_rank), c_int(kv_rank), c_int(rot_dim),
           c_int(rotary_dim), _ptr(q_weight), _ptr(kv_weight if write_kv else None), _ptr(inv_freq if write_kv and rotary_dim else None),
           _ptr(positions if write_kv else None), _ptr(token_seq if write_kv else None), _ptr(block_table if write_kv else None),
-          c_int(table_stride), _ptr(key_pages if write_kv else None), _ptr(cq_out), c_int(_code(cq_out.dtype)), c_float(eps),
+          c_int(table_stride), _ptr(key_pages if write_kv else None), _ptr(value_pages if write_kv else None), _ptr(cq_out),
+          c_int(_code(cq_out.dtype)), c_float(eps),
           c_int(tokens), c_int(block_size), c_int(num_blocks), c_int(1 if write_kv else 0), _stream())
     return cq_out
 
@@ -1494,15 +1501,73 @@ def latent_query_pack(q: Tensor, qa: Tensor, inv_freq: Tensor | None, positions:
     return out
 
 
-def latent_attention(q: Tensor, key_pages: Tensor, out: Tensor, cu_q: Tensor, ctx_len: Tensor, block_table: Tensor, *,
-                     num_seqs: int, max_q_len: int, heads: int, row_dim: int, value_dim: int, scale: float,
-                     num_decode: int | None = None, max_ctx: int | None = None) -> Tensor:
-    """Causal attention of ``heads`` query heads over one shared cache of keys only, ``key_pages`` [blocks, 1,
-    block_size, row_dim]: a row is the key of every head and its first ``value_dim`` dims are the value.  q
-    [T, heads * row_dim], out [T, heads * value_dim]; scores and softmax float32."""
-    return masked_attention(q, key_pages, None, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
-                            q_heads=heads, kv_heads=1, head_dim=row_dim, value_dim=value_dim, scale=scale,
-                            num_decode=num_decode, max_ctx=max_ctx)
+LATENT_TARGET_BLOCKS = 512      # blocks the matrix-core attention over a latent aims at before it stops cutting the keys into runs
+
+
+def latent_splits(num_seqs: int, max_q_len: int, heads: int, max_ctx: int | None) -> int:
+    """Runs that the matrix-core attention over a latent cuts every block's keys into: 1 when the step fills
+    the chip or the context is not known, else enough for about LATENT_TARGET_BLOCKS blocks with at least
+    four tiles of 32 keys each."""
+    if max_ctx is None:
+        return 1
+    blocks = -(-max(1, max_q_len) * heads // 64) * max(1, num_seqs)
+    return max(1, min(-(-LATENT_TARGET_BLOCKS // blocks), max_ctx // 128, 32))
+
+
+def latent_attention_supported(dtype, row_dim: int, value_dim: int, block_size: int) -> bool:
+    """Whether the matrix-core kernel takes these sizes (else the vector-ALU kernel does)."""
+    if dtype != torch.bfloat16 or block_size < 8 or block_size % 8:
+        return False
+    fn = library.load("attention_latent").fe_latent_attention_supported
+    fn.restype = c_int
+    return bool(fn(c_int(row_dim), c_int(value_dim)))
+
+
+def latent_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor | None, out: Tensor, cu_q: Tensor, ctx_len: Tensor,
+                     block_table: Tensor, *, num_seqs: int, max_q_len: int, heads: int, row_dim: int, value_dim: int,
+                     scale: float, num_decode: int | None = None, max_ctx: int | None = None, splits: int | None = None) -> Tensor:
+    """Causal attention of ``heads`` query heads over one shared cache of rows, ``key_pages`` [blocks, 1,
+    block_size, row_dim]: a row is the key of every head and its first ``value_dim`` dims are the value, which
+    ``value_pages`` [blocks, 1, value_dim, block_size] holds a second time, transposed (None: a cache of keys
+    only, read by the vector-ALU kernel).  q [T, heads * row_dim], out [T, heads * value_dim]; scores and
+    softmax float32.  bfloat16 at the sizes the matrix-core kernel is compiled for goes there (``splits``: its
+    key runs, chosen here if None); everything else, and the float32 mode, to the vector-ALU kernel."""
+    _gpu(q, "q")
+    _gpu(key_pages, "key_pages", q.dtype)
+    block_size = key_pages.shape[2] if key_pages.dim() == 4 else 0
+    if value_pages is None or not latent_attention_supported(q.dtype, row_dim, value_dim, block_size) or q.data_ptr() % 16:
+        return masked_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
+                                q_heads=heads, kv_heads=1, head_dim=row_dim, value_dim=value_dim, scale=scale,
+                                num_decode=num_decode, max_ctx=max_ctx)
+    _gpu(value_pages, "value_pages", q.dtype)
+    _gpu(out, "out", q.dtype)
+    _gpu(cu_q, "cu_q", torch.int32)
+    _gpu(ctx_len, "ctx_len", torch.int32)
+    _gpu(block_table, "block_table", torch.int32)
+    tokens = q.shape[0]
+    if q.shape != (tokens, heads * row_dim) or out.shape != (tokens, heads * value_dim):
+        raise KernelError(f"q must be [T, {heads * row_dim}] and out [T, {heads * value_dim}], got {tuple(q.shape)} and {tuple(out.shape)}")
+    if key_pages.dim() != 4 or key_pages.shape[1] != 1 or key_pages.shape[3] != row_dim:
+        raise KernelError(f"key pages must be [blocks, 1, block_size, {row_dim}], got {tuple(key_pages.shape)}")
+    num_blocks = key_pages.shape[0]
+    if value_pages.shape != (num_blocks, 1, value_dim, block_size):
+        raise KernelError(f"value pages are transposed: [blocks, 1, {value_dim}, block_size], got {tuple(value_pages.shape)}")
+    if cu_q.numel() != num_seqs + 1 or ctx_len.numel() != num_seqs or block_table.dim() != 2 or block_table.shape[0] < num_seqs \
+            or block_table.stride(1) != 1 or max_q_len < 1:
+        raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
+    if splits is None:
+        splits = latent_splits(num_seqs, max_q_len, heads, max_ctx)
+    if not 1 <= splits <= 64:
+        raise KernelError("between 1 and 64 key runs")
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((splits, tokens * heads, value_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((splits, tokens * heads, 2), dtype=torch.float32, device=q.device)
+    _call("attention_latent", "fe_latent_attention", _ptr(q), c_longlong(q.stride(0)), _ptr(key_pages), _ptr(value_pages), _ptr(out),
+          _ptr(part_o), _ptr(part_ml), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
+          c_int(max_q_len), c_int(heads), c_int(row_dim), c_int(value_dim), c_int(block_size), c_int(num_blocks), c_float(scale),
+          c_int(splits), c_int(tokens), _stream())
+    return out
 
 
 def heads_product(x: Tensor, weight: Tensor) -> Tensor:

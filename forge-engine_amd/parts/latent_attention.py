@@ -15,7 +15,9 @@ Keys and values are never made.  ``q_plain . W_uk[h] c = (W_uk[h]^T q_plain) . c
 query is taken through its key up-projection once and attention then runs over the cached rows
 ``[c | r]`` themselves, all heads sharing them like the query heads of one key/value head; the values
 are the first ``kv_rank`` dims of those rows, and ``W_uv[h]`` is applied once to the attention's
-result.  The cache holds keys only, ``kv_rank + rot_dim`` numbers a token.
+result.  The cache holds one row ``[c | r]`` a token as its key pages and ``c`` a second time in
+transposed value pages (the layout the matrix-core kernel reads its second operand in):
+``2 kv_rank + rot_dim`` numbers a token, whatever the number of heads.
 
 A layer with ``own_kv`` False has no ``W_dkv``: it is scheduled to read the pages of an earlier layer
 of the same geometry, with its own queries, ``W_uk``, ``W_uv`` and ``W_o``.
@@ -116,7 +118,7 @@ class LatentAttention(Mixer):
             raise KeyError(name)
 
     def cache_needs(self) -> CacheNeeds:
-        return CacheNeeds(paged=PagedKV(1, self.row_dim, None, 0))      # keys only: a row is its own value
+        return CacheNeeds(paged=PagedKV(1, self.row_dim, None, self.kv_rank))
 
     def forward(self, x: Tensor, batch, cache: CacheView, writes_cache: bool = True) -> Tensor:
         if writes_cache != self.own_kv:
@@ -127,7 +129,7 @@ class LatentAttention(Mixer):
         down = ops.linear(x, self.down_weight, out_dtype=torch.float32)
         latent_q = torch.empty((tokens, self.q_rank), dtype=x.dtype, device=x.device)
         ops.latent_norm_rope_write(down, self.q_norm, self.kv_norm, inv_freq, batch.positions, batch.token_seq,
-                                   cache.block_table, cache.key_pages, latent_q, q_rank=self.q_rank, kv_rank=self.kv_rank,
+                                   cache.block_table, cache.key_pages, cache.value_pages, latent_q, q_rank=self.q_rank, kv_rank=self.kv_rank,
                                    rot_dim=self.rot_dim, rotary_dim=rotary_dim, eps=self.eps, write_kv=writes_cache)
         q = ops.linear(latent_q, self.uq_weight)                                       # [T, H * (plain | rotated)]
         through_keys = ops.heads_product(q.view(tokens, heads, self.q_head)[:, :, :self.head_dim], self.uk)    # [H, T, kv_rank]
@@ -135,7 +137,7 @@ class LatentAttention(Mixer):
         ops.latent_query_pack(q, through_keys, inv_freq, batch.positions, rows, heads=heads, dim=self.head_dim,
                               rot_dim=self.rot_dim, rotary_dim=rotary_dim, kv_rank=self.kv_rank)
         read = torch.empty((tokens, heads * self.kv_rank), dtype=x.dtype, device=x.device)
-        ops.latent_attention(rows.view(tokens, heads * self.row_dim), cache.key_pages, read, batch.cu_q, batch.ctx_len,
+        ops.latent_attention(rows.view(tokens, heads * self.row_dim), cache.key_pages, cache.value_pages, read, batch.cu_q, batch.ctx_len,
                              cache.block_table, num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, heads=heads,
                              row_dim=self.row_dim, value_dim=self.kv_rank, scale=self.scale, num_decode=batch.num_decode,
                              max_ctx=batch.max_ctx)
@@ -147,7 +149,7 @@ class LatentAttention(Mixer):
         return self.position.token_inputs()
 
     def kernel_libraries(self):
-        return {"latent", "attention_masked", "stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+        return {"latent", "attention_latent", "attention_masked", "stream_ops", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
 
 
 register_part("mixer", "latent_attention", LatentAttention)

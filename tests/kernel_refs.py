@@ -735,8 +735,8 @@ def _turn(r, positions, inv_freq, rotary_dim):
     return torch.cat((lo * cos - hi * sin, hi * cos + lo * sin, r[..., rotary_dim:]), dim=-1)
 
 
-def latent_norm_rope_write(x, q_weight, kv_weight, inv_freq, positions, token_seq, block_table, key_pages, cq_out, *, q_rank,
-                           kv_rank, rot_dim, rotary_dim, eps, write_kv):
+def latent_norm_rope_write(x, q_weight, kv_weight, inv_freq, positions, token_seq, block_table, key_pages, value_pages, cq_out, *,
+                           q_rank, kv_rank, rot_dim, rotary_dim, eps, write_kv):
     x = x.float()
     cq_out.copy_((_unit(x[:, :q_rank], eps) * q_weight).to(cq_out.dtype))
     if not write_kv:
@@ -750,6 +750,8 @@ def latent_norm_rope_write(x, q_weight, kv_weight, inv_freq, positions, token_se
         page = int(block_table[int(token_seq[t]), pos // block_size])
         assert page >= 0, "token without a page"
         key_pages[page, 0, pos % block_size] = rows[t]
+        if value_pages is not None:
+            value_pages[page, 0, :, pos % block_size] = rows[t, :kv_rank]
     return cq_out
 
 
@@ -761,8 +763,8 @@ def latent_query_pack(q, qa, inv_freq, positions, out, *, heads, dim, rot_dim, r
     return out
 
 
-def latent_attention(q, key_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, heads, row_dim, value_dim, scale,
-                     num_decode=None, max_ctx=None):
+def latent_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len, heads, row_dim, value_dim,
+                     scale, num_decode=None, max_ctx=None, splits=None):
     block_size = key_pages.shape[2]
     for s in range(num_seqs):
         a, b = int(cu_q[s]), int(cu_q[s + 1])
@@ -770,11 +772,12 @@ def latent_attention(q, key_pages, out, cu_q, ctx_len, block_table, *, num_seqs,
         if b == a:
             continue
         rows = gather_pages(key_pages, block_table[s], ctx, block_size)[0]            # [ctx, row_dim]
+        values = rows[:, :value_dim] if value_pages is None else gather_pages(value_pages.transpose(2, 3), block_table[s], ctx, block_size)[0]
         for i in range(b - a):
             p = ctx - (b - a) + i
             queries = q[a + i].float().view(heads, row_dim)
             weights = torch.softmax(queries @ rows[:p + 1].T * scale, dim=-1)         # [heads, p + 1]
-            out[a + i] = (weights @ rows[:p + 1, :value_dim]).reshape(-1).to(out.dtype)
+            out[a + i] = (weights @ values[:p + 1]).reshape(-1).to(out.dtype)
     return out
 
 
