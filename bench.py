@@ -112,7 +112,7 @@ def parse_args():
     parser.add_argument("--points", default=None, help="other decode batch sizes to report")
     parser.add_argument("--widths", default="1024,2048,4096",
                         help="--phase design: model widths at which Mazanex and Qwen3 are measured side by side")
-    parser.add_argument("--design", choices=("mazanex", "rekezen", "malusun"), default="mazanex",
+    parser.add_argument("--design", choices=("mazanex", "rekezen", "malusun", "dubizen"), default="mazanex",
                         help="--phase design: which design is measured beside Qwen3")
     parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro", "check", "design"), default="all",
                         help="run one phase only (for profiles); the record then holds that phase alone")
@@ -351,11 +351,40 @@ def malusun_configs(width: int, layers: int) -> dict:
     return {"Malusun": malusun, "Rekezen": others["Rekezen"], "Qwen3": others["Qwen3"]}
 
 
-DESIGN_CONFIGS = {"mazanex": design_configs, "rekezen": rekezen_configs, "malusun": malusun_configs}
+def dubizen_configs(width: int, layers: int) -> dict:
+    """Dubizen beside Rekezen (the closest existing model: attention over the general path, layers that read an
+    earlier layer's cache, layer norms, a mixture of experts beside a shared one) and Qwen3, at one width: heads of
+    128, the same vocabulary and layer count.  Dubizen cycles through attention over a latent (a cached row of 512
+    + 64 numbers a token, queries through a bottleneck of 3/8 of the width, 64 rotated dims a head) with the dense
+    feed-forward of three widths, attention over a window of 1,024 in groups of four with biases by distance and
+    eight experts as wide as the model of which a token takes two out of the two best of four groups, beside a
+    gated shared one, and a layer that reads the first one's cache with the same experts."""
+    heads = max(4, width // 128)
+    latent = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": max(128, 3 * width // 8), "kv_rank": 512,
+              "scale": 192 ** -0.5, "rot": {"dims": 64, "base": 10000.0}}
+    windowed = {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
+                "bias_max": 512.0, "bias_rows": 32}
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 2, "scale": 2.5, "groups": {"count": 4, "keep": 2}}, "expert": {"ff": width},
+           "shared": {"ff": width}}
+
+    def entry(index):
+        if index % 3 == 0:
+            return {"type": "latent_attention", "mixer": latent, "mlp": {"kind": "dense", "ff": 3 * width}}
+        if index % 3 == 1:
+            return {"type": "attention", "mixer": windowed, "mlp": moe}
+        return {"type": "latent_attention", "mixer": dict(latent, kv_from=index - 2), "mlp": moe}
+
+    dubizen = {"architecture": "Dubizen", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+               "layers": [entry(i) for i in range(layers)]}
+    others = rekezen_configs(width, layers)
+    return {"Dubizen": dubizen, "Rekezen": others["Rekezen"], "Qwen3": others["Qwen3"]}
+
+
+DESIGN_CONFIGS = {"mazanex": design_configs, "rekezen": rekezen_configs, "malusun": malusun_configs, "dubizen": dubizen_configs}
 
 
 def design_comparison(args) -> int:
-    """Prefill and decode throughput of Mazanex (or, with ``--design``, Rekezen or Malusun) beside the closest existing models at equal
+    """Prefill and decode throughput of Mazanex (or, with ``--design``, Rekezen, Malusun or Dubizen) beside the closest existing models at equal
     width, layer count, feed-forward size and vocabulary; random weights, one JSON line a model and width."""
     import torch
 
