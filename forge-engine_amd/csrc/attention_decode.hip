@@ -100,14 +100,15 @@ struct Prepare {
 
 // MODE 0: finished queries; 1: PREPARE from the projection's bfloat16 output; 2: PREPARE from its
 // float32 partial sums.
-template <int D, int MODE, bool CAP = false, bool SLOPE = false>
+template <int D, int MODE, bool CAP = false, int DIST = 0>
 __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* key_pages,
     const bf16_t* value_pages, bf16_t* __restrict__ out, long long out_stride,
     float* part_o, float* part_ml, int* __restrict__ counters, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const int* __restrict__ block_table, int table_stride,
     int kv_heads, int groups, int block_shift, int num_blocks, int window, float scale_log2,
-    Prepare prep, int chunk, const float* __restrict__ sink, float cap_ratio, const float* __restrict__ slopes) {
+    Prepare prep, int chunk, const float* __restrict__ sink, float cap_ratio, const float* __restrict__ slopes,
+    int bias_span) {
   constexpr bool PREPARE = MODE != 0, FROM_SUMS = MODE == 2;
   const int block_size = 1 << block_shift, block_mask = block_size - 1;
   constexpr int KC = D / 32;        // MFMA k-steps over the head dim (scores)
@@ -135,9 +136,12 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lq = lane >> 4;
-  // SLOPE: head g's score of key j, after the scale, loses slopes[g] * (ctx - 1 - j); here in base-2 units
+  // DIST 1: head g's score of key j, after the scale, loses slopes[g] * (ctx - 1 - j); here in base-2 units.
+  // DIST 2: it gains table[g][min(ctx - 1 - j, span - 1)] instead, `slopes` being the table, float32 [heads][span]
   float slope2 = 0.f;
-  if constexpr (SLOPE) slope2 = (lr < groups ? slopes[hk * groups + lr] : 0.f) * 1.4426950408889634f;
+  if constexpr (DIST == 1) slope2 = (lr < groups ? slopes[hk * groups + lr] : 0.f) * 1.4426950408889634f;
+  const float* bias_row = nullptr;
+  if constexpr (DIST == 2) bias_row = slopes + (size_t)(hk * groups + min(lr, groups - 1)) * bias_span;
 
   // Everything that depends on nothing but the sequence's length is requested before any of it
   // is used, every load unconditional (out-of-range indices read a valid address and the value is
@@ -267,7 +271,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       if constexpr (CAP)
         raw = cap_ratio * (1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(raw * (2.f * 1.4426950408889634f / cap_ratio)) + 1.f));
       float v = raw * scale_log2;
-      if constexpr (SLOPE) v -= slope2 * (float)(ctx - 1 - key);
+      if constexpr (DIST == 1) v -= slope2 * (float)(ctx - 1 - key);
+      if constexpr (DIST == 2) v += bias_row[min(max(ctx - 1 - key, 0), bias_span - 1)] * 1.4426950408889634f;
       s[j] = (key >= k_begin && key < cached) ? v : -INFINITY;
       mx = fmaxf(mx, s[j]);
     }
@@ -582,10 +587,12 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
                          const int* cu_q, const int* ctx_len, const int* block_table, int table_stride,
                          int num_seqs, int kv_heads, int groups, int head_dim, int block_size,
                          int num_blocks, int window, float scale, int splits, const Prepare* prep,
-                         int chunk, const float* sink, hipStream_t stream, float softcap = 0.f, const float* slopes = nullptr) {
+                         int chunk, const float* sink, hipStream_t stream, float softcap = 0.f, const float* slopes = nullptr,
+                         int bias_span = 0) {
   if (num_seqs <= 0) return FE_OK;
   if (softcap < 0.f || (softcap > 0.f && (prep || !(scale > 0.f)))) return FE_BAD_ARGUMENT;
   if (slopes && (prep || softcap > 0.f)) return FE_BAD_ARGUMENT;
+  if (bias_span < 0 || (bias_span > 0 && !slopes)) return FE_BAD_ARGUMENT;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256) return FE_BAD_ARGUMENT;
   if (groups < 1 || groups > GMAX || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
   if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
@@ -602,16 +609,24 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
 #define FE_GO(DD, MODE)                                                                                    \
   paged_decode_kernel<DD, MODE><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, MODE ? *prep : none, chunk, sink, 0.f, nullptr)
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, MODE ? *prep : none, chunk, sink, 0.f, nullptr, 0)
 #define FE_GO_CAPPED(DD)                                                                                   \
   paged_decode_kernel<DD, 0, true><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, none, chunk, sink, softcap / scale, nullptr)
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, none, chunk, sink, softcap / scale, nullptr, 0)
 #define FE_GO_SLOPED(DD)                                                                                   \
-  paged_decode_kernel<DD, 0, false, true><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+  paged_decode_kernel<DD, 0, false, 1><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, none, chunk, sink, 0.f, slopes)
-  if (slopes) {
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, none, chunk, sink, 0.f, slopes, 0)
+#define FE_GO_TABLE(DD)                                                                                    \
+  paged_decode_kernel<DD, 0, false, 2><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, none, chunk, sink, 0.f, slopes, bias_span)
+  if (slopes && bias_span > 0) {
+    if (head_dim == 64) FE_GO_TABLE(64);
+    else if (head_dim == 128) FE_GO_TABLE(128);
+    else FE_GO_TABLE(256);
+  } else if (slopes) {
     if (head_dim == 64) FE_GO_SLOPED(64);
     else if (head_dim == 128) FE_GO_SLOPED(128);
     else FE_GO_SLOPED(256);
@@ -635,6 +650,7 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
 #undef FE_GO
 #undef FE_GO_CAPPED
 #undef FE_GO_SLOPED
+#undef FE_GO_TABLE
   return fe_check_launch();
 }
 
@@ -701,6 +717,22 @@ extern "C" int fe_paged_attention_decode_sloped(const void* q, long long q_strid
   return launch_decode(q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
                        ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
                        num_blocks, window, scale, splits, nullptr, chunk, sink, stream, 0.f, slopes);
+}
+
+// The same with a bias by distance: head h's score of key j, after the scale, gains table[h][min(ctx - 1 - j, span - 1)]
+// (table: float32 [kv_heads * groups][span]).
+extern "C" int fe_paged_attention_decode_biased(const void* q, long long q_stride, const void* key_pages,
+                                                const void* value_pages, void* out, long long out_stride,
+                                                float* part_o, float* part_ml, int* counters, const int* cu_q,
+                                                const int* ctx_len, const int* block_table, int table_stride,
+                                                int num_seqs, int kv_heads, int groups, int head_dim,
+                                                int block_size, int num_blocks, int window, int chunk,
+                                                const float* sink, const float* table, int span, float scale, int splits,
+                                                hipStream_t stream) {
+  if (!table || span < 1) return FE_BAD_ARGUMENT;
+  return launch_decode(q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
+                       ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
+                       num_blocks, window, scale, splits, nullptr, chunk, sink, stream, 0.f, table, span);
 }
 
 // The same for a batch in which EVERY sequence brings one token, straight from the fused

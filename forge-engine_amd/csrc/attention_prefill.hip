@@ -133,14 +133,14 @@ __device__ __forceinline__ int wave_most(int v) {
   return __builtin_amdgcn_readfirstlane(max((int)r[0], (int)r[1]));
 }
 
-template <int D, int KG, int RM, bool CAP = false, bool SLOPE = false>
+template <int D, int KG, int RM, bool CAP = false, int DIST = 0>
 __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_kernel(   // RM = 1: four waves a SIMD (128 registers), RM = 2: two
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int block_shift, int num_blocks, int window,
     float scale_log2, int num_seqs, int heads_per_xcd, int chunk, const float* __restrict__ sink, float cap_ratio,
-    const float* __restrict__ slopes) {
+    const float* __restrict__ slopes, int bias_span) {
   const int block_mask = (1 << block_shift) - 1;
   constexpr int BM = 64 * RM;
   constexpr int KC = D / 32;            // MFMA k-steps over the head dim (scores)
@@ -381,8 +381,16 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
   };
   // SLOPE: a penalty on distance, slope_h * (position - key), comes off the score after the scale: off the raw
   // score it is that times 1 / scale (what it does to keys that the masks hide does not matter).
+  // DIST 2: a bias by distance, table[head][min(position - key, span - 1)] (`slopes` being the table, float32
+  // [heads][span]), joins the score after the scale: to the raw score it is that times 1 / scale.
   float slope_raw = 0.f;
-  if constexpr (SLOPE) slope_raw = slopes[head] * 1.4426950408889634f / scale_log2;
+  if constexpr (DIST == 1) slope_raw = slopes[head] * 1.4426950408889634f / scale_log2;
+  const float* bias_row = nullptr;
+  float bias_raw = 0.f;
+  if constexpr (DIST == 2) {
+    bias_row = slopes + (size_t)head * bias_span;
+    bias_raw = 1.4426950408889634f / scale_log2;
+  }
   auto slope_scores = [&](int key_base, floatx4 (&st)[RM][2][2]) {
 #pragma unroll
     for (int rm = 0; rm < RM; ++rm) {
@@ -392,9 +400,19 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
         st[rm][j >> 3][(j >> 2) & 1][j & 3] -= slope_raw * (nearest - (float)(32 * (j >> 3) + (j & 7)));
     }
   };
+  auto bias_scores = [&](int key_base, floatx4 (&st)[RM][2][2]) {
+#pragma unroll
+    for (int rm = 0; rm < RM; ++rm) {
+      const int nearest = row_pos[rm] - key_base - 8 * lq;
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        st[rm][j >> 3][(j >> 2) & 1][j & 3] += bias_raw * bias_row[min(max(nearest - (32 * (j >> 3) + (j & 7)), 0), bias_span - 1)];
+    }
+  };
   auto softmax = [&](int key_base, floatx4 (&st)[RM][2][2], uintx4 (&pw)[RM][2]) {
     if constexpr (CAP) cap_scores(st);
-    if constexpr (SLOPE) slope_scores(key_base, st);
+    if constexpr (DIST == 1) slope_scores(key_base, st);
+    if constexpr (DIST == 2) bias_scores(key_base, st);
     if (is_edge(key_base)) mask_edges(key_base, st);
 #pragma unroll
     for (int rm = 0; rm < RM; ++rm)
@@ -668,7 +686,7 @@ static int launch_prefill_sloped(const void* q, long long q_stride, const void* 
                                  long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
                                  int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
                                  int block_size, int num_blocks, int window, int chunk, const float* sink, float scale,
-                                 float softcap, const float* slopes, int key_groups, int row_sets, int total_q, hipStream_t stream);
+                                 float softcap, const float* slopes, int key_groups, int row_sets, int total_q, hipStream_t stream, int bias_span = 0);
 static int launch_prefill(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
                           long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
                           int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
@@ -732,6 +750,21 @@ extern "C" int fe_paged_attention_prefill_sloped(const void* q, long long q_stri
                                scale, 0.f, slopes, key_groups, row_sets, total_q, stream);
 }
 
+// The same with a bias by distance: head h's score of key j, after the scale, gains table[h][min(position - j, span - 1)]
+// (table: float32 [kv_heads * groups][span]).
+extern "C" int fe_paged_attention_prefill_biased(const void* q, long long q_stride, const void* key_pages,
+                                                 const void* value_pages, void* out, long long out_stride,
+                                                 const int* cu_q, const int* ctx_len, const int* block_table,
+                                                 int table_stride, int num_seqs, int max_q_len, int kv_heads,
+                                                 int groups, int head_dim, int block_size, int num_blocks,
+                                                 int window, int chunk, const float* sink, const float* table, int span, float scale,
+                                                 int key_groups, int row_sets, int total_q, hipStream_t stream) {
+  if (!table || span < 1 || !(scale > 0.f)) return FE_BAD_ARGUMENT;
+  return launch_prefill_sloped(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len, block_table, table_stride,
+                               num_seqs, max_q_len, kv_heads, groups, head_dim, block_size, num_blocks, window, chunk, sink,
+                               scale, 0.f, table, key_groups, row_sets, total_q, stream, span);
+}
+
 static int launch_prefill(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
                           long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
                           int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
@@ -746,9 +779,9 @@ static int launch_prefill_sloped(const void* q, long long q_stride, const void* 
                                  long long out_stride, const int* cu_q, const int* ctx_len, const int* block_table,
                                  int table_stride, int num_seqs, int max_q_len, int kv_heads, int groups, int head_dim,
                                  int block_size, int num_blocks, int window, int chunk, const float* sink, float scale,
-                                 float softcap, const float* slopes, int key_groups, int row_sets, int total_q, hipStream_t stream) {
+                                 float softcap, const float* slopes, int key_groups, int row_sets, int total_q, hipStream_t stream, int bias_span) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
-  if (chunk < 0 || (slopes && softcap > 0.f)) return FE_BAD_ARGUMENT;
+  if (chunk < 0 || (slopes && softcap > 0.f) || bias_span < 0 || (bias_span > 0 && !slopes)) return FE_BAD_ARGUMENT;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
   if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
   if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1 || q_stride % 8 || out_stride % 4) return FE_BAD_ARGUMENT;
@@ -785,12 +818,13 @@ static int launch_prefill_sloped(const void* q, long long q_stride, const void* 
 #define FE_GO_C(DD, GG, RR, CC, SS)                                                                                  \
   paged_prefill_kernel<DD, GG, RR, CC, SS><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
-      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd, chunk, sink, cap_ratio, slopes)
+      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd, chunk, sink, cap_ratio, slopes, bias_span)
 #define FE_GO(DD, GG, RR)                                 \
   do {                                                    \
-    if (softcap > 0.f) FE_GO_C(DD, GG, RR, true, false);  \
-    else if (slopes) FE_GO_C(DD, GG, RR, false, true);    \
-    else FE_GO_C(DD, GG, RR, false, false);               \
+    if (softcap > 0.f) FE_GO_C(DD, GG, RR, true, 0);      \
+    else if (slopes && bias_span > 0) FE_GO_C(DD, GG, RR, false, 2); \
+    else if (slopes) FE_GO_C(DD, GG, RR, false, 1);       \
+    else FE_GO_C(DD, GG, RR, false, 0);                   \
   } while (0)
 #define FE_GO_D(DD)                                          \
   if (key_groups == 1 && row_sets == 1) FE_GO(DD, 1, 1);      \

@@ -714,7 +714,8 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
                     window: int | None = None, num_decode: int | None = None,
                     max_ctx: int | None = None, splits: int | None = None, chunk: int | None = None,
-                    sink: Tensor | None = None, softcap: float | None = None, slopes: Tensor | None = None) -> Tensor:
+                    sink: Tensor | None = None, softcap: float | None = None, slopes: Tensor | None = None,
+                    dist_bias: Tensor | None = None) -> Tensor:
     """Attention of every query token of a mixed batch over its paged keys.
 
     ``chunk`` (a token reads keys of its own run of that many positions only), ``sink``
@@ -766,8 +767,13 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                   and q.data_ptr() % 16 == 0 and q_stride % 8 == 0)      # the fast kernels read 16 bytes at a time
     fast_decode = bf16_pages and head_dim in (64, 128, 256) and groups <= 8
     fast_prefill = bf16_pages and head_dim in (64, 128)
-    masked = chunk is not None or sink is not None or softcap is not None or slopes is not None
+    masked = chunk is not None or sink is not None or softcap is not None or slopes is not None or dist_bias is not None
     if masked:
+        if dist_bias is not None:     # a table of biases by distance, float32 [Hq, span]: entry min(position - j, span - 1) joins the score
+            _gpu(dist_bias, "dist_bias", torch.float32)
+            if dist_bias.dim() != 2 or dist_bias.shape[0] != q_heads or dist_bias.shape[1] < 1 or slopes is not None or softcap is not None \
+                    or not scale > 0.0:
+                raise KernelError(f"dist_bias must be [{q_heads}, span], with a positive scale and without slopes or a soft cap")
         if slopes is not None:
             _gpu(slopes, "slopes", torch.float32)
             if slopes.shape != (q_heads,) or softcap is not None or not scale > 0.0:
@@ -807,8 +813,10 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
             part_ml = torch.empty(num_seqs * kv_heads * splits * groups * 2, dtype=torch.float32, device=q.device)
             counters = _split_counters(q.device, num_seqs * kv_heads)
         mask = (c_int(chunk or 0), _ptr(sink)) + ((_ptr(slopes),) if slopes is not None else ()) if masked else ()
+        if dist_bias is not None:
+            mask = (c_int(chunk or 0), _ptr(sink), _ptr(dist_bias), c_int(dist_bias.shape[1]))
         cap = (c_float(softcap),) if softcap is not None else ()
-        name = ("fe_paged_attention_decode_sloped" if slopes is not None else "fe_paged_attention_decode_capped" if cap
+        name = ("fe_paged_attention_decode_biased" if dist_bias is not None else "fe_paged_attention_decode_sloped" if slopes is not None else "fe_paged_attention_decode_capped" if cap
                 else "fe_paged_attention_decode_masked" if masked else "fe_paged_attention_decode")
         _call("attention_decode", name, _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(part_o),
@@ -817,8 +825,10 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               c_int(num_blocks), c_int(window or 0), *mask, c_float(scale), *cap, c_int(splits), _stream())
     if any_longer and fast_prefill:
         mask = (c_int(chunk or 0), _ptr(sink)) + ((_ptr(slopes),) if slopes is not None else ()) if masked else ()
+        if dist_bias is not None:
+            mask = (c_int(chunk or 0), _ptr(sink), _ptr(dist_bias), c_int(dist_bias.shape[1]))
         cap = (c_float(softcap),) if softcap is not None else ()
-        name = ("fe_paged_attention_prefill_sloped" if slopes is not None else "fe_paged_attention_prefill_capped" if cap
+        name = ("fe_paged_attention_prefill_biased" if dist_bias is not None else "fe_paged_attention_prefill_sloped" if slopes is not None else "fe_paged_attention_prefill_capped" if cap
                 else "fe_paged_attention_prefill_masked" if masked else "fe_paged_attention_prefill")
         _call("attention_prefill", name, _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
@@ -1397,11 +1407,13 @@ def masked_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor | None, o
     if (window is not None and window < 1) or (chunk is not None and chunk < 1) or max_q_len < 1:
         raise KernelError("window, chunk and max_q_len must be positive")
     if (q.dtype == torch.bfloat16 and head_dim == value_dim and head_dim in (64, 128) and q_heads // kv_heads <= 8
-            and not (slopes is not None and softcap is not None) and dist_bias is None and value_pages is not None
+            and not (slopes is not None and softcap is not None) and value_pages is not None
+            and not (dist_bias is not None and (slopes is not None or softcap is not None))
             and block_size >= 16 and block_size & (block_size - 1) == 0 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0):
         paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, num_seqs=num_seqs, max_q_len=max_q_len,
                         q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window,
-                        num_decode=num_decode, max_ctx=max_ctx, chunk=chunk, sink=sink, softcap=softcap, slopes=slopes)
+                        num_decode=num_decode, max_ctx=max_ctx, chunk=chunk, sink=sink, softcap=softcap, slopes=slopes,
+                        dist_bias=dist_bias)
         if gate is not None:
             _call("stream_ops", "fe_sigmoid_gate", _ptr(out), _ptr(gate), c_longlong(gate_stride), c_int(_code(out.dtype)),
                   c_int(tokens), c_int(q_heads * value_dim), c_int(value_dim if head_gate else 1), _stream())
