@@ -7,8 +7,12 @@
 //
 // Block = 4 waves on 64 query rows of one sequence, a row being a (token, head) pair, token-major, so
 // that the 64 rows of a block share their keys; a wave owns 16 rows.  Keys are walked in tiles of 32:
-// the tile's keys go through LDS (all four waves read them), the values come straight from their
-// transposed pages into the MFMA operands.  S^T = K Q^T and O^T = V^T P^T on MFMA 16x16x32 with
+// the tile's keys and its transposed values reach LDS by `global_load_lds_dwordx4` (64 lanes x 16 bytes at
+// consecutive LDS addresses, no staging registers: every load of a tile is in flight at once), and all
+// four waves read their MFMA operands from there.  Which global bytes a lane loads is free, where they
+// land is not, so a key row's 16-byte chunks lie permuted by the row's low bits and a value dim's four
+// key chunks by the dim's bits 2 and 3: the operand reads of 16 lanes then spread over the banks.  Where two
+// blocks fit a CU, one block's loads run under the other's products.  S^T = K Q^T and O^T = V^T P^T on MFMA 16x16x32 with
 // scores, statistics and outputs in registers: lane (r = lane % 16, g = lane / 16) holds, of row r,
 // the scores of keys 8g .. 8g + 7 of the tile (the key rows of the first product are permuted so that
 // they come out that way, which is the order the second product's operands want) and the outputs of
@@ -32,18 +36,31 @@ __device__ __forceinline__ unsigned int pack_two(float lo, float hi) {
   return (unsigned int)float_to_bf16(lo) | ((unsigned int)float_to_bf16(hi) << 16);
 }
 
+__device__ __forceinline__ void tile_to_lds(const void* global, void* lds) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)global,
+                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
+// Queries (DK / 8 registers a lane) and outputs (DV / 4) stay in registers for the whole walk: the sizes that need
+// more than half a SIMD's registers for them run one block a CU, the others two.
 template <int DK, int DV>
-__global__ __launch_bounds__(256) void latent_attention_kernel(
+__global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_attention_kernel(
     const bf16_t* __restrict__ q, size_t q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
     const int* __restrict__ block_table, int table_stride, int heads, int block_size, int num_blocks,
     float scale_log2, int splits, int total_rows) {
   constexpr int KC = DK / 32, DT = DV / 16, CHUNKS = DK / 8;
-  constexpr int KS = DK + 8;           // a key's row in LDS, elements: 16 bytes of padding against bank conflicts
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[LA_KEYS * KS];
+  constexpr int SW = CHUNKS % 8 == 0 ? 7 : (CHUNKS % 4 == 0 ? 3 : 1);     // a key row's chunks are permuted by row & SW
+  constexpr int K_UNITS = LA_KEYS * CHUNKS, V_UNITS = DV * 4;             // 16-byte units of a tile's keys and values
+  constexpr int LOADS = (K_UNITS + V_UNITS) / 64;                         // load instructions a tile, 64 units each
+  static_assert(K_UNITS % 64 == 0 && V_UNITS % 64 == 0, "whole load instructions");
+  extern __shared__ __attribute__((aligned(16))) unsigned char tile_lds[];
+  const bf16_t* Ks = (const bf16_t*)tile_lds;                             // unit u: key u / CHUNKS, chunk (u % CHUNKS) ^ (key & SW)
+  const bf16_t* Vs = (const bf16_t*)(tile_lds + K_UNITS * 16);            // unit u: dim u / 4, keys 8 ((u % 4) ^ (dim >> 2 & 3)) .. + 7
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, lq = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, lr = lane & 15, lq = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int seq = blockIdx.z, split = blockIdx.y;
   const int q0 = cu_q[seq];
   const int q_len = cu_q[seq + 1] - q0;
@@ -77,21 +94,37 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
   for (int t = 0; t < DT; ++t) o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
   const int* table = block_table + (size_t)seq * table_stride;
+  const int last_key = ctx - 1;
 
   for (int tile = t_lo; tile < t_hi; ++tile) {
     const int kb = tile * LA_KEYS;
     __syncthreads();        // the tile before is consumed
-    for (int idx = tid; idx < LA_KEYS * CHUNKS; idx += 256) {
-      const int key = idx / CHUNKS, chunk = idx - key * CHUNKS;
-      const int kp = kb + key;
-      uintx4 v = uintx4{0u, 0u, 0u, 0u};
-      if (kp < ctx) {
-        const int page = table[kp / block_size];
-        if (page >= 0 && page < num_blocks)
-          v = *(const uintx4*)(key_pages + ((size_t)page * block_size + kp % block_size) * DK + chunk * 8);
+    // the wave's share of the tile's loads; keys beyond the context read the last key's page (their scores are
+    // masked and their values cleared in the operand), so every address is a valid one
+#pragma unroll
+    for (int n = 0; n < (LOADS + 3) / 4; ++n) {
+      const int load = wave + 4 * n;
+      if (load < LOADS) {
+        const int u = load * 64 + lane;
+        const bf16_t* src;
+        if (load < K_UNITS / 64) {
+          const int key = u / CHUNKS, slot = u - key * CHUNKS;
+          const int kp = min(kb + key, last_key);
+          int page = table[kp / block_size];
+          page = min(max(page, 0), num_blocks - 1);
+          src = key_pages + ((size_t)page * block_size + kp % block_size) * DK + (slot ^ (key & SW)) * 8;
+        } else {
+          const int uv = u - K_UNITS;
+          const int dim = uv >> 2, kc = (uv & 3) ^ ((dim >> 2) & 3);
+          const int kp = min(kb + 8 * kc, last_key & ~7);
+          int page = table[kp / block_size];
+          page = min(max(page, 0), num_blocks - 1);
+          src = value_pages + ((size_t)page * DV + dim) * block_size + kp % block_size;
+        }
+        tile_to_lds(src, tile_lds + load * 1024);
       }
-      *(uintx4*)(Ks + key * KS + chunk * 8) = v;
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (!wave_ok || kb > wave_pos_max) continue;      // the whole wave: no row, or no row that sees this tile
 
@@ -100,10 +133,11 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     for (int h = 0; h < 2; ++h) {
       st[h] = floatx4{0.f, 0.f, 0.f, 0.f};
       // operand row lr of half h is key 8 (lr / 4) + 4 h + lr % 4, so that result row 4 g + i is key 8 g + 4 h + i
-      const bf16_t* krow = Ks + (8 * (lr >> 2) + 4 * h + (lr & 3)) * KS + lq * 8;
+      const int key = 8 * (lr >> 2) + 4 * h + (lr & 3);
+      const bf16_t* krow = Ks + (size_t)key * DK;
 #pragma unroll
       for (int c = 0; c < KC; ++c)
-        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(krow + c * 32), qb[c], st[h], 0, 0, 0);
+        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(krow + ((c * 4 + lq) ^ (key & SW)) * 8), qb[c], st[h], 0, 0, 0);
     }
     float s[8];
     float mx = -INFINITY;
@@ -128,22 +162,19 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     m_run = m_new;
     const bf16x8 pb = __builtin_bit_cast(bf16x8, uintx4{pack_two(s[0], s[1]), pack_two(s[2], s[3]), pack_two(s[4], s[5]), pack_two(s[6], s[7])});
 
-    // this lane's eight keys of the value operand: one page (pages hold a multiple of eight slots)
+    // this lane's eight keys of the value operand: those beyond the context are cleared
     const int vkey = kb + 8 * lq;
-    int vpage = vkey < ctx ? table[vkey / block_size] : -1;
-    const bool v_ok = vpage >= 0 && vpage < num_blocks;
-    if (!v_ok) vpage = 0;
     uintx4 v_mask;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const unsigned int lo = (v_ok && vkey + 2 * w < ctx) ? 0x0000ffffu : 0u;
-      const unsigned int hi = (v_ok && vkey + 2 * w + 1 < ctx) ? 0xffff0000u : 0u;
+      const unsigned int lo = vkey + 2 * w < ctx ? 0x0000ffffu : 0u;
+      const unsigned int hi = vkey + 2 * w + 1 < ctx ? 0xffff0000u : 0u;
       v_mask[w] = lo | hi;
     }
-    const bf16_t* vbase = value_pages + (size_t)vpage * DV * block_size + (vkey % block_size) + (size_t)lr * block_size;
+    const bf16_t* vrow = Vs + ((size_t)lr * 4 + (lq ^ ((lr >> 2) & 3))) * 8;
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-      const uintx4 va = *(const uintx4*)(vbase + (size_t)t * 16 * block_size) & v_mask;
+      const uintx4 va = *(const uintx4*)(vrow + (size_t)t * 16 * 32) & v_mask;
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[t][i] *= corr;
       o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, va), pb, o[t], 0, 0, 0);
@@ -200,7 +231,14 @@ static int launch_latent(const void* q, long long q_stride, const void* key_page
                          float scale, int splits, int tokens, hipStream_t stream) {
   const long long rows = (long long)max_q_len * heads;
   const dim3 grid((unsigned)((rows + LA_ROWS - 1) / LA_ROWS), splits, num_seqs);
-  latent_attention_kernel<DK, DV><<<grid, 256, 0, stream>>>(
+  constexpr int lds = (LA_KEYS * DK + DV * 32) * 2;       // a tile's keys and its transposed values
+  static bool sized = false;                              // more than 64 KB of LDS a block has to be asked for, once a kernel
+  if (lds > 64 * 1024 && !sized) {
+    if (hipFuncSetAttribute((const void*)latent_attention_kernel<DK, DV>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return FE_LAUNCH_FAILED;
+    sized = true;
+  }
+  latent_attention_kernel<DK, DV><<<grid, 256, lds, stream>>>(
       (const bf16_t*)q, (size_t)q_stride, (const bf16_t*)key_pages, (const bf16_t*)value_pages, (bf16_t*)out, part_o,
       part_ml, cu_q, ctx_len, block_table, table_stride, heads, block_size, num_blocks, scale * 1.4426950408889634f,
       splits, tokens * heads);
