@@ -11,8 +11,8 @@
 // consecutive LDS addresses, no staging registers: every load of a tile is in flight at once), and all
 // four waves read their MFMA operands from there.  Which global bytes a lane loads is free, where they
 // land is not, so a key row's 16-byte chunks lie permuted by the row's low bits and a value dim's four
-// key chunks by the dim's bits 2 and 3: the operand reads of 16 lanes then spread over the banks.  Where two
-// blocks fit a CU, one block's loads run under the other's products.  S^T = K Q^T and O^T = V^T P^T on MFMA 16x16x32 with
+// key chunks by the dim's bits 2 and 3: the operand reads of 16 lanes then spread over the banks.  Two
+// buffers: a tile's loads run under the products of the tile before.  S^T = K Q^T and O^T = V^T P^T on MFMA 16x16x32 with
 // scores, statistics and outputs in registers: lane (r = lane % 16, g = lane / 16) holds, of row r,
 // the scores of keys 8g .. 8g + 7 of the tile (the key rows of the first product are permuted so that
 // they come out that way, which is the order the second product's operands want) and the outputs of
@@ -36,6 +36,40 @@ __device__ __forceinline__ unsigned int pack_two(float lo, float hi) {
   return (unsigned int)float_to_bf16(lo) | ((unsigned int)float_to_bf16(hi) << 16);
 }
 
+// Where chunk `slot` of key row `key` lies in the row's LDS image (and the other way round: the map is its
+// own inverse).  The 16 rows that one operand read touches are rows 8a + b (+ 4h), a and b below 4; rows are
+// CHUNKS units of 16 bytes apart, which moves odd rows by 8 units mod 16 where CHUNKS is 8 mod 16, and
+// 4a + b with its bit 3 flipped for odd b, XORed into the chunk index, puts the 16 rows on 16 distinct
+// units mod 16, that is on all banks once.  A row's last chunks, where they do not fill a group of 16, are
+// permuted within their own group of 8 (or 4) only.
+template <int CHUNKS>
+__device__ __forceinline__ int key_chunk(int key, int slot) {
+  constexpr int WHOLE = CHUNKS & ~15, REST = CHUNKS & 15;
+  constexpr int REST_MASK = REST % 8 == 0 ? 7 : (REST % 4 == 0 ? 3 : (REST % 2 == 0 ? 1 : 0));
+  int s = ((key >> 3) & 3) * 4 + (key & 3);
+  if (CHUNKS % 16 == 8) s ^= (key & 1) << 3;
+  return slot ^ (slot < WHOLE ? s : (s & REST_MASK));
+}
+
+// 16 bytes from the LDS byte address `at`; nothing waits for them here
+__device__ __forceinline__ uintx4 lds_read16(unsigned int at) {
+  uintx4 v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(at) : "memory");
+  return v;
+}
+// wait until at most `pending` of this wave's LDS reads are outstanding; `v` is what the wait is for (LDS reads
+// return in order; whatever else is under way on the same counter makes such a wait stricter, never weaker)
+template <int PENDING>
+__device__ __forceinline__ void lds_arrived(uintx4& v) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(PENDING));
+}
+#define LA_AHEAD 4      // operand reads in flight ahead of the product that uses them
+#define LA_RING 8
+__device__ __forceinline__ void lds_wait(uintx4& v, int pending) {
+  if (pending >= 4) lds_arrived<4>(v); else if (pending == 3) lds_arrived<3>(v); else if (pending == 2) lds_arrived<2>(v);
+  else if (pending == 1) lds_arrived<1>(v); else lds_arrived<0>(v);
+}
+
 __device__ __forceinline__ void tile_to_lds(const void* global, void* lds) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)global,
                                    (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
@@ -48,16 +82,18 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
     const bf16_t* __restrict__ q, size_t q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
-    const int* __restrict__ block_table, int table_stride, int heads, int block_size, int num_blocks,
+    const int* __restrict__ block_table, int table_stride, int heads, int block_shift, int num_blocks,
     float scale_log2, int splits, int total_rows) {
   constexpr int KC = DK / 32, DT = DV / 16, CHUNKS = DK / 8;
-  constexpr int SW = CHUNKS % 8 == 0 ? 7 : (CHUNKS % 4 == 0 ? 3 : 1);     // a key row's chunks are permuted by row & SW
   constexpr int K_UNITS = LA_KEYS * CHUNKS, V_UNITS = DV * 4;             // 16-byte units of a tile's keys and values
   constexpr int LOADS = (K_UNITS + V_UNITS) / 64;                         // load instructions a tile, 64 units each
+  constexpr int MINE = (LOADS + 3) / 4;                                   // ... of which a wave issues this many
+  constexpr int TILE_BYTES = (K_UNITS + V_UNITS) * 16;                    // one buffer
+  static_assert(DT >= LA_AHEAD && 2 * KC >= LA_AHEAD, "the rings of operand reads");
   static_assert(K_UNITS % 64 == 0 && V_UNITS % 64 == 0, "whole load instructions");
   extern __shared__ __attribute__((aligned(16))) unsigned char tile_lds[];
-  const bf16_t* Ks = (const bf16_t*)tile_lds;                             // unit u: key u / CHUNKS, chunk (u % CHUNKS) ^ (key & SW)
-  const bf16_t* Vs = (const bf16_t*)(tile_lds + K_UNITS * 16);            // unit u: dim u / 4, keys 8 ((u % 4) ^ (dim >> 2 & 3)) .. + 7
+  // a buffer: K_UNITS units of keys (unit u: key u / CHUNKS, chunk key_chunk(key, u % CHUNKS) of it), then V_UNITS units of
+  // values (unit u: dim u / 4, keys 8 ((u % 4) ^ (dim >> 2 & 3)) .. + 7 of the tile)
 
   const int tid = threadIdx.x, lane = tid & 63, lr = lane & 15, lq = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -96,48 +132,87 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
   const int* table = block_table + (size_t)seq * table_stride;
   const int last_key = ctx - 1;
 
-  for (int tile = t_lo; tile < t_hi; ++tile) {
-    const int kb = tile * LA_KEYS;
-    __syncthreads();        // the tile before is consumed
-    // the wave's share of the tile's loads; keys beyond the context read the last key's page (their scores are
-    // masked and their values cleared in the operand), so every address is a valid one
+  // One tile's loads: the wave's share of them.  Keys beyond the context read the last key's page (their
+  // scores are masked and their values cleared in the operand), so every address is a valid one.  What does
+  // not change from tile to tile is worked out once: which key of the tile a lane's load n fetches and where
+  // in that key's row (or value dim) it starts.  The page ids of a tile are fetched a tile ahead, behind the
+  // loads of the tile before: a wait for a page id right before its load would stall every tile.
+  const int block_size = 1 << block_shift, slot_mask = block_size - 1;
+  int rel[MINE], off[MINE], lim[MINE], page_id[MINE];
 #pragma unroll
-    for (int n = 0; n < (LOADS + 3) / 4; ++n) {
+  for (int n = 0; n < MINE; ++n) {
+    const int load = min(wave + 4 * n, LOADS - 1);
+    const int u = load * 64 + lane;
+    if (load < K_UNITS / 64) {
+      const int key = u / CHUNKS, slot = u - key * CHUNKS;
+      rel[n] = key;
+      off[n] = key_chunk<CHUNKS>(key, slot) * 8;
+      lim[n] = last_key;
+    } else {
+      const int uv = u - K_UNITS;
+      const int dim = uv >> 2, kc = (uv & 3) ^ ((dim >> 2) & 3);
+      rel[n] = 8 * kc;
+      off[n] = dim << block_shift;
+      lim[n] = last_key & ~7;
+    }
+  }
+  auto page_ids = [&](int tile) {
+#pragma unroll
+    for (int n = 0; n < MINE; ++n) page_id[n] = table[min(tile * LA_KEYS + rel[n], lim[n]) >> block_shift];
+  };
+  auto fetch = [&](int tile, int buffer) {
+    const int kb = tile * LA_KEYS;
+#pragma unroll
+    for (int n = 0; n < MINE; ++n) {
       const int load = wave + 4 * n;
       if (load < LOADS) {
-        const int u = load * 64 + lane;
-        const bf16_t* src;
-        if (load < K_UNITS / 64) {
-          const int key = u / CHUNKS, slot = u - key * CHUNKS;
-          const int kp = min(kb + key, last_key);
-          int page = table[kp / block_size];
-          page = min(max(page, 0), num_blocks - 1);
-          src = key_pages + ((size_t)page * block_size + kp % block_size) * DK + (slot ^ (key & SW)) * 8;
-        } else {
-          const int uv = u - K_UNITS;
-          const int dim = uv >> 2, kc = (uv & 3) ^ ((dim >> 2) & 3);
-          const int kp = min(kb + 8 * kc, last_key & ~7);
-          int page = table[kp / block_size];
-          page = min(max(page, 0), num_blocks - 1);
-          src = value_pages + ((size_t)page * DV + dim) * block_size + kp % block_size;
-        }
-        tile_to_lds(src, tile_lds + load * 1024);
+        const int kp = min(kb + rel[n], lim[n]);
+        const size_t page = (size_t)min(max(page_id[n], 0), num_blocks - 1);
+        const bf16_t* src = load < K_UNITS / 64 ? key_pages + ((page << block_shift) + (kp & slot_mask)) * DK + off[n]
+                                                : value_pages + ((page * DV) << block_shift) + off[n] + (kp & slot_mask);
+        tile_to_lds(src, tile_lds + buffer * TILE_BYTES + load * 1024);
       }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (!wave_ok || kb > wave_pos_max) continue;      // the whole wave: no row, or no row that sees this tile
+  };
+  const unsigned int lds_at = (unsigned int)(size_t)(const __attribute__((address_space(3))) unsigned char*)tile_lds;
 
-    floatx4 st[2];
+  // Two buffers: a tile's loads are issued before the tile before it is multiplied, and land meanwhile.  The
+  // operands are read from LDS by inline assembly with their waits written out: the compiler, with loads
+  // into LDS in flight, would wait for all of them before its first LDS read.
+  if (t_lo < t_hi) {
+    page_ids(t_lo);
+    fetch(t_lo, 0);
+    page_ids(t_lo + 1);
+  }
+  for (int tile = t_lo; tile < t_hi; ++tile) {
+    const int kb = tile * LA_KEYS;
+    const int buffer = (tile - t_lo) & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's loads of the tile have landed
+    __syncthreads();                                        // ... and everyone's; the other buffer's tile is consumed
+    if (tile + 1 < t_hi) {
+      fetch(tile + 1, buffer ^ 1);
+      page_ids(tile + 2);         // keys beyond the context read the last key's entry: always a valid index
+    }
+    if (!wave_ok || kb > wave_pos_max) continue;            // the whole wave: no row, or no row that sees this tile
+    const unsigned int keys_at = lds_at + buffer * TILE_BYTES, values_at = keys_at + K_UNITS * 16;
+
+    // S^T: operand row lr of half h is key 8 (lr / 4) + 4 h + lr % 4, so that result row 4 g + i is key 8 g + 4 h + i
+    floatx4 st[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    {
+      constexpr int FRAGMENTS = 2 * KC;       // step c outermost, half h inside
+      auto fragment = [&](int f) -> uintx4 {
+        const int key = 8 * (lr >> 2) + 4 * (f & 1) + (lr & 3);
+        return lds_read16(keys_at + (unsigned int)((key * CHUNKS + key_chunk<CHUNKS>(key, (f >> 1) * 4 + lq)) * 16));
+      };
+      uintx4 ring[LA_RING];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      st[h] = floatx4{0.f, 0.f, 0.f, 0.f};
-      // operand row lr of half h is key 8 (lr / 4) + 4 h + lr % 4, so that result row 4 g + i is key 8 g + 4 h + i
-      const int key = 8 * (lr >> 2) + 4 * h + (lr & 3);
-      const bf16_t* krow = Ks + (size_t)key * DK;
+      for (int f = 0; f < LA_AHEAD; ++f) ring[f] = fragment(f);
 #pragma unroll
-      for (int c = 0; c < KC; ++c)
-        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(krow + ((c * 4 + lq) ^ (key & SW)) * 8), qb[c], st[h], 0, 0, 0);
+      for (int f = 0; f < FRAGMENTS; ++f) {
+        if (f + LA_AHEAD < FRAGMENTS) ring[(f + LA_AHEAD) % LA_RING] = fragment(f + LA_AHEAD);
+        lds_wait(ring[f % LA_RING], FRAGMENTS - 1 - f < LA_AHEAD ? FRAGMENTS - 1 - f : LA_AHEAD);
+        st[f & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ring[f % LA_RING]), qb[f >> 1], st[f & 1], 0, 0, 0);
+      }
     }
     float s[8];
     float mx = -INFINITY;
@@ -162,7 +237,7 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
     m_run = m_new;
     const bf16x8 pb = __builtin_bit_cast(bf16x8, uintx4{pack_two(s[0], s[1]), pack_two(s[2], s[3]), pack_two(s[4], s[5]), pack_two(s[6], s[7])});
 
-    // this lane's eight keys of the value operand: those beyond the context are cleared
+    // O^T: this lane's eight keys of the value operand, those beyond the context cleared
     const int vkey = kb + 8 * lq;
     uintx4 v_mask;
 #pragma unroll
@@ -171,13 +246,23 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
       const unsigned int hi = vkey + 2 * w + 1 < ctx ? 0xffff0000u : 0u;
       v_mask[w] = lo | hi;
     }
-    const bf16_t* vrow = Vs + ((size_t)lr * 4 + (lq ^ ((lr >> 2) & 3))) * 8;
+    const bool rescale = __builtin_amdgcn_ballot_w64(corr != 1.f) != 0;      // the whole wave: once the maxima have settled, nothing to do
+    {
+      const unsigned int mine = values_at + (unsigned int)((lr * 4 + (lq ^ ((lr >> 2) & 3))) * 16);
+      auto fragment = [&](int t) -> uintx4 { return lds_read16(mine + (unsigned int)(t * 16 * 64)); };
+      uintx4 ring[LA_RING];
 #pragma unroll
-    for (int t = 0; t < DT; ++t) {
-      const uintx4 va = *(const uintx4*)(vrow + (size_t)t * 16 * 32) & v_mask;
+      for (int t = 0; t < LA_AHEAD; ++t) ring[t] = fragment(t);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[t][i] *= corr;
-      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, va), pb, o[t], 0, 0, 0);
+      for (int t = 0; t < DT; ++t) {
+        if (t + LA_AHEAD < DT) ring[(t + LA_AHEAD) % LA_RING] = fragment(t + LA_AHEAD);
+        if (rescale) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[t][i] *= corr;
+        }
+        lds_wait(ring[t % LA_RING], DT - 1 - t < LA_AHEAD ? DT - 1 - t : LA_AHEAD);
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ring[t % LA_RING] & v_mask), pb, o[t], 0, 0, 0);
+      }
     }
   }
 
@@ -231,16 +316,18 @@ static int launch_latent(const void* q, long long q_stride, const void* key_page
                          float scale, int splits, int tokens, hipStream_t stream) {
   const long long rows = (long long)max_q_len * heads;
   const dim3 grid((unsigned)((rows + LA_ROWS - 1) / LA_ROWS), splits, num_seqs);
-  constexpr int lds = (LA_KEYS * DK + DV * 32) * 2;       // a tile's keys and its transposed values
+  constexpr int lds = 2 * (LA_KEYS * DK + DV * 32) * 2;   // two buffers of a tile's keys and its transposed values
   static bool sized = false;                              // more than 64 KB of LDS a block has to be asked for, once a kernel
   if (lds > 64 * 1024 && !sized) {
     if (hipFuncSetAttribute((const void*)latent_attention_kernel<DK, DV>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return FE_LAUNCH_FAILED;
     sized = true;
   }
+  int block_shift = 0;
+  while ((1 << block_shift) < block_size) ++block_shift;
   latent_attention_kernel<DK, DV><<<grid, 256, lds, stream>>>(
       (const bf16_t*)q, (size_t)q_stride, (const bf16_t*)key_pages, (const bf16_t*)value_pages, (bf16_t*)out, part_o,
-      part_ml, cu_q, ctx_len, block_table, table_stride, heads, block_size, num_blocks, scale * 1.4426950408889634f,
+      part_ml, cu_q, ctx_len, block_table, table_stride, heads, block_shift, num_blocks, scale * 1.4426950408889634f,
       splits, tokens * heads);
   if (splits > 1) latent_merge_kernel<<<tokens * heads, 128, 0, stream>>>(part_o, part_ml, (bf16_t*)out, splits, tokens * heads, DV);
   return fe_check_launch();
@@ -258,7 +345,7 @@ extern "C" int fe_latent_attention(const void* q, long long q_stride, const void
                                    int row_dim, int value_dim, int block_size, int num_blocks, float scale, int splits,
                                    int tokens, hipStream_t stream) {
   if (tokens <= 0 || num_seqs <= 0) return FE_OK;
-  if (heads < 1 || max_q_len < 1 || block_size < 8 || block_size % 8 || num_blocks < 1 || splits < 1 || splits > 64 ||
+  if (heads < 1 || max_q_len < 1 || block_size < 8 || (block_size & (block_size - 1)) || num_blocks < 1 || splits < 1 || splits > 64 ||
       num_seqs > 65535 || q_stride < (long long)heads * row_dim || q_stride % 8 || (splits > 1 && (!part_o || !part_ml)) ||
       (long long)tokens * heads > 0x7fffffffLL || !fe_latent_attention_supported(row_dim, value_dim))
     return FE_BAD_ARGUMENT;

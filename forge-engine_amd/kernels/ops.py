@@ -1528,7 +1528,7 @@ def latent_splits(num_seqs: int, max_q_len: int, heads: int, max_ctx: int | None
 
 def latent_attention_supported(dtype, row_dim: int, value_dim: int, block_size: int) -> bool:
     """Whether the matrix-core kernel takes these sizes (else the vector-ALU kernel does)."""
-    if dtype != torch.bfloat16 or block_size < 8 or block_size % 8:
+    if dtype != torch.bfloat16 or block_size < 8 or block_size & (block_size - 1):      # pages of a power of two, eight slots or more
         return False
     fn = library.load("attention_latent").fe_latent_attention_supported
     fn.restype = c_int
