@@ -51,10 +51,12 @@ __device__ __forceinline__ int key_chunk(int key, int slot) {
   return slot ^ (slot < WHOLE ? s : (s & REST_MASK));
 }
 
-// 16 bytes from the LDS byte address `at`; nothing waits for them here
+// 16 bytes from the LDS byte address `at` + OFFSET (an immediate of the instruction); nothing waits for them here
+template <int OFFSET>
 __device__ __forceinline__ uintx4 lds_read16(unsigned int at) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "the instruction's offset field");
   uintx4 v;
-  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(at) : "memory");
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(at), "n"(OFFSET) : "memory");
   return v;
 }
 // wait until at most `pending` of this wave's LDS reads are outstanding; `v` is what the wait is for (LDS reads
@@ -65,9 +67,27 @@ __device__ __forceinline__ void lds_arrived(uintx4& v) {
 }
 #define LA_AHEAD 4      // operand reads in flight ahead of the product that uses them
 #define LA_RING 8
-__device__ __forceinline__ void lds_wait(uintx4& v, int pending) {
-  if (pending >= 4) lds_arrived<4>(v); else if (pending == 3) lds_arrived<3>(v); else if (pending == 2) lds_arrived<2>(v);
-  else if (pending == 1) lds_arrived<1>(v); else lds_arrived<0>(v);
+
+// body(integral constant I) for I = FROM .. TO - 1: a loop whose counter is a constant expression in its body
+template <int I> struct index_constant { static constexpr int value = I; };
+template <int FROM, int TO, typename Body>
+__device__ __forceinline__ void static_for(Body&& body) {
+  if constexpr (FROM < TO) {
+    body(index_constant<FROM>{});
+    static_for<FROM + 1, TO>(body);
+  }
+}
+
+// Fragment F of the first product's key operand (step F / 2 of the dims, half F % 2 of the tile's keys) from the
+// key image at LDS byte address `keys_at`.  The lane's chunk of step c is 4c + lq, at slot (4c + lq) ^ s of its
+// row, s below 16 and lq below 4: the slot is (4c & ~15) + ((4c & 15) ^ lq ^ s), so `at` holds, per half, the
+// row's byte offset plus 16 ((4j) ^ lq ^ s) for j = 0 .. 3 (entries 0 .. 3), and the same with s cut to the
+// row's last, smaller group of chunks (entries 4 .. 7); the rest is an immediate of the instruction.
+template <int CHUNKS, int F>
+__device__ __forceinline__ uintx4 key_fragment(unsigned int keys_at, const unsigned int (&at)[2][8]) {
+  constexpr int c = F >> 1, h = F & 1, first = 4 * c;
+  constexpr bool rest = first >= (CHUNKS & ~15);
+  return lds_read16<(first & ~15) * 16>(keys_at + at[h][(rest ? 4 : 0) + ((first & 15) >> 2)]);
 }
 
 __device__ __forceinline__ void tile_to_lds(const void* global, void* lds) {
@@ -103,7 +123,7 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
   const int ctx = ctx_len[seq];
   const int before = ctx - q_len;
   const int rows_total = q_len * heads;
-  const int row0 = blockIdx.x * LA_ROWS;
+  const int row0 = (gridDim.x - 1 - blockIdx.x) * LA_ROWS;      // a sequence's last rows walk the most keys: they start first
   if (row0 >= rows_total || before < 0) return;
 
   const int my_row = row0 + wave * 16 + lr;
@@ -175,6 +195,20 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
     }
   };
   const unsigned int lds_at = (unsigned int)(size_t)(const __attribute__((address_space(3))) unsigned char*)tile_lds;
+  // where this lane's operand reads start within a buffer (see key_fragment); operand row lr of half h is key
+  // 8 (lr / 4) + 4 h + lr % 4, so that result row 4 g + i is key 8 g + 4 h + i
+  unsigned int key_at[2][8];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int key = 8 * (lr >> 2) + 4 * h + (lr & 3);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      key_at[h][j] = (unsigned int)((key * CHUNKS + (key_chunk<CHUNKS>(key, 4 * j + lq) & 15)) * 16);
+      const int r = 4 * j + lq < (CHUNKS & 15) ? 4 * j + lq : 0;        // entries beyond the row's last group are never read
+      key_at[h][4 + j] = (unsigned int)((key * CHUNKS + (key_chunk<CHUNKS>(key, (CHUNKS & ~15) + r) & 15)) * 16);
+    }
+  }
+  const unsigned int value_at = (unsigned int)((lr * 4 + (lq ^ ((lr >> 2) & 3))) * 16);
 
   // Two buffers: a tile's loads are issued before the tile before it is multiplied, and land meanwhile.  The
   // operands are read from LDS by inline assembly with their waits written out: the compiler, with loads
@@ -196,23 +230,17 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
     if (!wave_ok || kb > wave_pos_max) continue;            // the whole wave: no row, or no row that sees this tile
     const unsigned int keys_at = lds_at + buffer * TILE_BYTES, values_at = keys_at + K_UNITS * 16;
 
-    // S^T: operand row lr of half h is key 8 (lr / 4) + 4 h + lr % 4, so that result row 4 g + i is key 8 g + 4 h + i
     floatx4 st[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
     {
       constexpr int FRAGMENTS = 2 * KC;       // step c outermost, half h inside
-      auto fragment = [&](int f) -> uintx4 {
-        const int key = 8 * (lr >> 2) + 4 * (f & 1) + (lr & 3);
-        return lds_read16(keys_at + (unsigned int)((key * CHUNKS + key_chunk<CHUNKS>(key, (f >> 1) * 4 + lq)) * 16));
-      };
       uintx4 ring[LA_RING];
-#pragma unroll
-      for (int f = 0; f < LA_AHEAD; ++f) ring[f] = fragment(f);
-#pragma unroll
-      for (int f = 0; f < FRAGMENTS; ++f) {
-        if (f + LA_AHEAD < FRAGMENTS) ring[(f + LA_AHEAD) % LA_RING] = fragment(f + LA_AHEAD);
-        lds_wait(ring[f % LA_RING], FRAGMENTS - 1 - f < LA_AHEAD ? FRAGMENTS - 1 - f : LA_AHEAD);
+      static_for<0, LA_AHEAD>([&](auto f) { ring[f.value] = key_fragment<CHUNKS, f.value>(keys_at, key_at); });
+      static_for<0, FRAGMENTS>([&](auto fc) {
+        constexpr int f = fc.value;
+        if constexpr (f + LA_AHEAD < FRAGMENTS) ring[(f + LA_AHEAD) % LA_RING] = key_fragment<CHUNKS, f + LA_AHEAD>(keys_at, key_at);
+        lds_arrived<(FRAGMENTS - 1 - f < LA_AHEAD ? FRAGMENTS - 1 - f : LA_AHEAD)>(ring[f % LA_RING]);
         st[f & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ring[f % LA_RING]), qb[f >> 1], st[f & 1], 0, 0, 0);
-      }
+      });
     }
     float s[8];
     float mx = -INFINITY;
@@ -237,32 +265,35 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
     m_run = m_new;
     const bf16x8 pb = __builtin_bit_cast(bf16x8, uintx4{pack_two(s[0], s[1]), pack_two(s[2], s[3]), pack_two(s[4], s[5]), pack_two(s[6], s[7])});
 
-    // O^T: this lane's eight keys of the value operand, those beyond the context cleared
-    const int vkey = kb + 8 * lq;
-    uintx4 v_mask;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const unsigned int lo = vkey + 2 * w < ctx ? 0x0000ffffu : 0u;
-      const unsigned int hi = vkey + 2 * w + 1 < ctx ? 0xffff0000u : 0u;
-      v_mask[w] = lo | hi;
-    }
+    // O^T: this lane's eight keys of the value operand; in the tile that crosses the context's end those
+    // beyond it are cleared
     const bool rescale = __builtin_amdgcn_ballot_w64(corr != 1.f) != 0;      // the whole wave: once the maxima have settled, nothing to do
+    const bool crosses = kb + LA_KEYS > ctx;
+    uintx4 v_mask = uintx4{~0u, ~0u, ~0u, ~0u};
+    if (crosses) {
+      const int vkey = kb + 8 * lq;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const unsigned int lo = vkey + 2 * w < ctx ? 0x0000ffffu : 0u;
+        const unsigned int hi = vkey + 2 * w + 1 < ctx ? 0xffff0000u : 0u;
+        v_mask[w] = lo | hi;
+      }
+    }
     {
-      const unsigned int mine = values_at + (unsigned int)((lr * 4 + (lq ^ ((lr >> 2) & 3))) * 16);
-      auto fragment = [&](int t) -> uintx4 { return lds_read16(mine + (unsigned int)(t * 16 * 64)); };
+      const unsigned int mine = values_at + value_at;
       uintx4 ring[LA_RING];
-#pragma unroll
-      for (int t = 0; t < LA_AHEAD; ++t) ring[t] = fragment(t);
-#pragma unroll
-      for (int t = 0; t < DT; ++t) {
-        if (t + LA_AHEAD < DT) ring[(t + LA_AHEAD) % LA_RING] = fragment(t + LA_AHEAD);
+      static_for<0, LA_AHEAD>([&](auto t) { ring[t.value] = lds_read16<t.value * 1024>(mine); });
+      static_for<0, DT>([&](auto tc) {
+        constexpr int t = tc.value;
+        if constexpr (t + LA_AHEAD < DT) ring[(t + LA_AHEAD) % LA_RING] = lds_read16<(t + LA_AHEAD) * 1024>(mine);
         if (rescale) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) o[t][i] *= corr;
         }
-        lds_wait(ring[t % LA_RING], DT - 1 - t < LA_AHEAD ? DT - 1 - t : LA_AHEAD);
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ring[t % LA_RING] & v_mask), pb, o[t], 0, 0, 0);
-      }
+        lds_arrived<(DT - 1 - t < LA_AHEAD ? DT - 1 - t : LA_AHEAD)>(ring[t % LA_RING]);
+        if (crosses) ring[t % LA_RING] &= v_mask;
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ring[t % LA_RING]), pb, o[t], 0, 0, 0);
+      });
     }
   }
 
