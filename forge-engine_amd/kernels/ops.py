@@ -1514,16 +1514,18 @@ def latent_query_pack(q: Tensor, qa: Tensor, inv_freq: Tensor | None, positions:
 
 
 LATENT_TARGET_BLOCKS = 512      # blocks the matrix-core attention over a latent aims at before it stops cutting the keys into runs
+LATENT_MIN_TILES = 4            # ... and the fewest tiles a run may have (8 sequences at 1,024 keys, 16 heads, rows of 576, us a call with the
+                                # merge: 1 run 110, 2 runs 62, 4 runs 40, 8 runs 32, 16 runs 35, 32 runs 51)
 
 
 def latent_splits(num_seqs: int, max_q_len: int, heads: int, max_ctx: int | None) -> int:
     """Runs that the matrix-core attention over a latent cuts every block's keys into: 1 when the step fills
     the chip or the context is not known, else enough for about LATENT_TARGET_BLOCKS blocks with at least
-    four tiles of 32 keys each."""
+    LATENT_MIN_TILES tiles of 32 keys each."""
     if max_ctx is None:
         return 1
     blocks = -(-max(1, max_q_len) * heads // 64) * max(1, num_seqs)
-    return max(1, min(-(-LATENT_TARGET_BLOCKS // blocks), max_ctx // 128, 32))
+    return max(1, min(-(-LATENT_TARGET_BLOCKS // blocks), max_ctx // (32 * LATENT_MIN_TILES), 32))
 
 
 def latent_attention_supported(dtype, row_dim: int, value_dim: int, block_size: int) -> bool:
