@@ -7,7 +7,7 @@ width (``width``), the norms' epsilon (``norm.eps``), the factor on every normed
 feed-forward (``mlp``, or null for none).
 
 ``attention``: ``heads``, ``kv_heads``, ``dim``, ``vdim``, ``scale``, ``mask.size`` (the sliding
-window) and ``bias_max`` (the distance at which the table of biases by distance reaches its last
+window; absent: every earlier token is seen) and ``bias_max`` (the distance at which the table of biases by distance reaches its last
 row; the table's rows are the tensor's).  ``latent_attention``: ``heads``, ``dim``, ``rot_dim``,
 ``vdim``, ``q_rank``, ``kv_rank``, ``scale``, ``rot.dims``, ``rot.base`` and optionally ``kv_from``
 (an earlier layer with a down-projection of its own and the same ``kv_rank``, ``rot_dim`` and
@@ -15,7 +15,8 @@ rotation, whose cache this layer reads).  ``mlp``: ``kind`` ``dense`` with ``ff`
 ``moe`` with ``router.experts``, ``router.top``, ``router.scale``, optionally ``router.groups``
 (``count``, ``keep``), ``expert.ff`` and optionally ``shared.ff``.  The rows of a layer's table of
 biases by distance are nowhere in config.json: the checkpoint's tensor shapes give them
-(``with_tensor_shapes``), or ``mixer.bias_rows`` for a model without a checkpoint.
+(``with_tensor_shapes``), or ``mixer.bias_rows`` for a model without a checkpoint; a ``q_rank`` that
+config.json leaves out is read from the shapes as well.
 """
 
 from __future__ import annotations
@@ -47,15 +48,18 @@ def _check_attention(raw: dict, where: str) -> None:
     read.integer("vdim")
     read.number("scale")
     read.number("bias_max")
-    KeyReader(_section(raw, "mask", where)).integer("size")
+    if raw.get("mask") is not None:         # without it every earlier token is seen
+        KeyReader(_section(raw, "mask", where)).integer("size")
     if raw.get("bias_rows") is not None:
         read.integer("bias_rows", minimum=2)
 
 
 def _check_latent(raw: dict, where: str, index: int, layers: list) -> None:
     read = KeyReader(raw)
-    for key in ("heads", "dim", "vdim", "q_rank", "kv_rank"):
+    for key in ("heads", "dim", "vdim", "kv_rank"):
         read.integer(key)
+    if raw.get("q_rank") is not None:       # else the checkpoint's tensor shapes give it
+        read.integer("q_rank")
     rot_dim = read.integer("rot_dim", minimum=2)
     read.number("scale")
     rot = _section(raw, "rot", where)
@@ -144,12 +148,16 @@ class DubizenConfig(ModelConfig):
                    layers_json=json.dumps(layers, sort_keys=True), eos_token_id=eos)
 
     def with_tensor_shapes(self, shapes: dict[str, tuple[int, ...]]) -> "DubizenConfig":
-        """The rows of every layer's table of biases by distance, from the checkpoint's tensor shapes."""
+        """The rows of every layer's table of biases by distance (and a query bottleneck's width that
+        config.json does not give), from the checkpoint's tensor shapes."""
         layers = self.layers
         for index, layer in enumerate(layers):
             shape = shapes.get(f"l{index}.mix.rel")
             if layer["type"] == "attention" and shape is not None and len(shape) == 2:
                 layer["mixer"]["bias_rows"] = int(shape[0])
+            shape = shapes.get(f"l{index}.mix.dq")
+            if layer["type"] == "latent_attention" and layer["mixer"].get("q_rank") is None and shape is not None and len(shape) == 2:
+                layer["mixer"]["q_rank"] = int(shape[0])
         return replace(self, layers_json=json.dumps(layers, sort_keys=True))
 
     def to_dict(self) -> dict[str, Any]:

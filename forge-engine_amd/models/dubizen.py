@@ -23,6 +23,7 @@ shared expert (``.shared.*``) times ``sigmoid(.shared.sg . x)``.
 from __future__ import annotations
 
 from ..config.dubizen import DEFAULT_BIAS_ROWS, DubizenConfig
+from ..config.model import ConfigError
 from ..parts.plan import LayerCall, LayerSpec, ModelPlan, PartSpec
 from ..registry import register_architecture
 
@@ -37,11 +38,13 @@ def _mixer(config: DubizenConfig, kind: str, sizes: dict, prefix: str) -> PartSp
     if kind == "attention":
         return PartSpec("gqa_attention", {
             "hidden_size": config.width, "num_heads": sizes["heads"], "num_kv_heads": sizes["kv_heads"], "head_dim": sizes["dim"],
-            "value_dim": sizes["vdim"], "scale": sizes["scale"], "window": sizes["mask"]["size"], "bias": True, "bias_init": "small",
+            "value_dim": sizes["vdim"], "scale": sizes["scale"], "window": (sizes.get("mask") or {}).get("size"), "bias": True, "bias_init": "small",
             "qk_norm_eps": config.norm_eps, "position": PartSpec("none"), "force_general": True, "names": ATTENTION_NAMES,
             "distance_bias": {"rows": sizes.get("bias_rows") or DEFAULT_BIAS_ROWS, "reach": sizes["bias_max"]},
         }, prefix)
     rot = sizes["rot"]
+    if sizes.get("q_rank") is None:
+        raise ConfigError(f"{prefix}: neither config.json nor a checkpoint's shapes give the query bottleneck's width ('q_rank')")
     return PartSpec("latent_attention", {
         "hidden_size": config.width, "num_heads": sizes["heads"], "head_dim": sizes["dim"], "rot_dim": sizes["rot_dim"],
         "value_dim": sizes["vdim"], "q_rank": sizes["q_rank"], "kv_rank": sizes["kv_rank"], "scale": sizes["scale"],

@@ -66,10 +66,12 @@ class Residual:
         self.streams: Tensor | None = None
         self.pending_mix: tuple[Tensor, Tensor] | None = None    # (mix [S, S] indexed [from, to], share [S])
         self.pending_norm: tuple[Tensor, float] | None = None    # (weight, eps): the update is RMS-normed before it is added
+        self.in_compute_dtype: Tensor | None = None               # the stream as a norm of updates last stored it beside h (the same values)
 
     def add(self, update: Tensor | None) -> None:
         """Leave an update pending; None: the part has added it into the stream itself."""
         self.flush()
+        self.in_compute_dtype = None
         self.pending = update
 
     def add_normed(self, update: Tensor, weight: Tensor, eps: float) -> None:
@@ -78,6 +80,7 @@ class Residual:
         self.flush()
         if self.streams is not None:
             raise ValueError("a norm behind a sublayer needs a model with one residual stream")
+        self.in_compute_dtype = None
         self.pending, self.pending_norm = update, (weight, float(eps))
 
     def take_normed(self):
@@ -89,6 +92,7 @@ class Residual:
     def add_mixed(self, update: Tensor, mix: Tensor, share: Tensor) -> None:
         """Several streams: leave ``x_t <- sum_s mix[s, t] x_s + share[t] * update`` pending."""
         self.flush()
+        self.in_compute_dtype = None
         self.pending, self.pending_mix = update, (mix, share)
 
     def take_pending(self):
@@ -110,7 +114,14 @@ class Residual:
         """The stream with nothing pending, for a part that adds its update itself."""
         if self.streams is not None:
             raise ValueError("a part that adds into the stream itself needs a model with one stream")
+        self.in_compute_dtype = None
         return self.flush()
+
+    def stored(self, out: Tensor) -> Tensor:
+        """A norm of updates has just stored the new stream in the compute dtype as well (``out``): the next
+        sublayer that reads the stream itself takes that copy instead of casting the stream again."""
+        self.in_compute_dtype = out
+        return out
 
     def flush(self) -> Tensor:
         if self.pending is not None:

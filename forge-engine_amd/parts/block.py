@@ -81,8 +81,8 @@ class OutputNormBlock(Block):
                                 batch.state_slots, num_seqs=batch.num_seqs, out_dtype=self.ctx.dtype)[0]
             mixer_cache = dataclasses.replace(
                 cache, states={n: t for n, t in cache.states.items() if n != self.SHIFT_STATE})
-        else:
-            s = ops.cast_rows(h, self.ctx.dtype)
+        else:       # the layer before has left the stream in the compute dtype as well, unless this is the first
+            s = residual.in_compute_dtype if residual.in_compute_dtype is not None else ops.cast_rows(h, self.ctx.dtype)
             mixer_cache = cache
         residual.add(self.mixer.forward(s, batch, mixer_cache, writes_cache))
         x = self.norms["mixer_out"].forward(residual)

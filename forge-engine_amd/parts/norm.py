@@ -71,7 +71,7 @@ class UpdateRMSNorm(RMSNorm):
         if update is None:
             raise ValueError("a norm of updates needs a pending update")
         out = torch.empty((residual.h.shape[0], self.size), dtype=self.ctx.dtype, device=residual.h.device)
-        return ops.rmsnorm_update(residual.h, update, self.weight, self.eps, out)
+        return residual.stored(ops.rmsnorm_update(residual.h, update, self.weight, self.eps, out))
 
     def kernel_libraries(self):
         return {"rowwise", "stream_ops"}
@@ -154,7 +154,7 @@ class UpdateLayerNorm(Norm):
         if update is None:
             raise ValueError("a norm of updates needs a pending update")
         out = torch.empty((residual.h.shape[0], self.size), dtype=self.ctx.dtype, device=residual.h.device)
-        return ops.layernorm_update(residual.h, update, self.weight, self.eps, self.factor, out)
+        return residual.stored(ops.layernorm_update(residual.h, update, self.weight, self.eps, self.factor, out))
 
     def kernel_libraries(self):
         return {"stream_ops"}

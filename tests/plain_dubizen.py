@@ -76,7 +76,7 @@ def softmax_read(scores: torch.Tensor, visible: torch.Tensor, values: torch.Tens
 
 def windowed_attention(h, w, p, sizes: dict, eps: float, positions, state: dict | None = None) -> torch.Tensor:
     heads, kv_heads, dim, vdim = sizes["heads"], sizes["kv_heads"], sizes["dim"], sizes["vdim"]
-    window, scale, reach = sizes["mask"]["size"], sizes["scale"], sizes["bias_max"]
+    window, scale, reach = (sizes.get("mask") or {}).get("size"), sizes["scale"], sizes["bias_max"]     # no mask: every earlier token
     count = h.shape[0]
     q = (h @ w[p + ".q"].T + w[p + ".q.b"]).view(count, heads, dim)
     k = (h @ w[p + ".k"].T + w[p + ".k.b"]).view(count, kv_heads, dim)
@@ -92,7 +92,7 @@ def windowed_attention(h, w, p, sizes: dict, eps: float, positions, state: dict 
         state.update(k=k, v=v, positions=key_positions)
     table = w[p + ".rel"]
     distance = positions[:, None] - key_positions[None, :]
-    visible = (distance >= 0) & (distance < window)
+    visible = (distance >= 0) & (distance < (window if window is not None else distance.max() + 1))
     rows = torch.tensor([[distance_bucket(int(n), table.shape[0], reach) if n >= 0 else 0 for n in line] for line in distance.tolist()])
     out = torch.zeros((count, heads, vdim), dtype=F64)
     for head in range(heads):

@@ -204,7 +204,7 @@ def single(mixer, mlp, *, vocab=50, width=24, mult=0.5, before=None):
     return du.config(vocab, width, layers, mult=mult)
 
 
-@pytest.mark.parametrize("case", ["windowed", "windowed_one_kv_head", "latent", "latent_reader", "dense", "experts", "experts_all"])
+@pytest.mark.parametrize("case", ["windowed", "windowed_one_kv_head", "no_window", "latent", "latent_reader", "dense", "experts", "experts_all"])
 def test_each_mechanism_alone_through_the_engine(case, tmp_path, monkeypatch):
     """A model of one layer (two for a reader of another layer's cache) around the mechanism, in portions and
     single tokens through the engine, against the plain function for it."""
@@ -213,6 +213,7 @@ def test_each_mechanism_alone_through_the_engine(case, tmp_path, monkeypatch):
     raw = {
         "windowed": single(du.attention(6, 3, 10, 14, 5, reach=4.0, rows=4), None),
         "windowed_one_kv_head": single(du.attention(5, 1, 6, 2, 17, reach=60.0, rows=20), None),
+        "no_window": single(du.attention(2, 2, 6, 10, 1, reach=11.0, rows=6), None),      # the mask is taken out below: biases up to the table's reach and beyond
         "latent": single(du.latent(3, 10, 6, 14, 9, 11, turned=4, base=77.0), None),
         "latent_reader": single(du.latent(2, 6, 6, 4, 5, 11, turned=4, base=77.0, source=0), None,
                                 before=du.layer(du.latent(3, 10, 6, 14, 9, 11, turned=4, base=77.0), None)),
@@ -220,7 +221,14 @@ def test_each_mechanism_alone_through_the_engine(case, tmp_path, monkeypatch):
         "experts": single(quiet, du.moe(12, 3, 10, shared=6, groups=(4, 2), scale=2.5)),
         "experts_all": single(quiet, du.moe(3, 3, 10, scale=0.5)),
     }[case]
+    if case == "no_window":
+        del raw["layers"][0]["mixer"]["mask"]
     folder = du.write_model(raw, 5, tmp_path / "model")
+    if case == "latent":        # a config.json that leaves the query bottleneck's width to the tensors' shapes
+        import json
+        stored = json.loads((folder / "config.json").read_text())
+        del stored["layers"][0]["mixer"]["q_rank"]
+        (folder / "config.json").write_text(json.dumps(stored))
     requests = ru.make_requests({"vocab_size": raw["vocab"]}, 2, (33, 6))
     want = du.plain_logits(folder, requests)
     for trace in (ru.trace_portions(requests, sizes=(5, 2, 9, 3)), ru.trace_tail(requests, 12)):
