@@ -67,7 +67,8 @@ def test_activations_and_row_gates(dtype):
 
 
 @pytest.mark.parametrize("tokens,hidden,experts,top,groups,keep", [(1, 48, 6, 2, 2, 1), (37, 64, 9, 3, 3, 2), (150, 256, 16, 4, 4, 2), (70, 40, 4, 4, 1, 1),
-                                                                   (300, 128, 64, 8, 8, 3), (5, 32, 12, 1, 12, 5)])
+                                                                   (300, 128, 64, 8, 8, 3), (5, 32, 12, 1, 12, 5), (70, 64, 256, 8, 8, 4),
+                                                                   (129, 48, 192, 6, 16, 2)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_choice_of_experts_within_the_best_groups(tokens, hidden, experts, top, groups, keep, dtype):
     """Corrections of both signs; a router with one more row whose logits come back untouched; the choice and
