@@ -364,7 +364,7 @@ def dubizen_configs(width: int, layers: int) -> dict:
               "scale": 192 ** -0.5, "rot": {"dims": 64, "base": 10000.0}}
     windowed = {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
                 "bias_max": 512.0, "bias_rows": 32}
-    moe = {"kind": "moe", "router": {"experts": 8, "top": 2, "scale": 2.5, "groups": {"count": 4, "keep": 2}}, "expert": {"ff": width},
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}, "expert": {"ff": width},
            "shared": {"ff": width}}
 
     def entry(index):
@@ -374,7 +374,7 @@ def dubizen_configs(width: int, layers: int) -> dict:
             return {"type": "attention", "mixer": windowed, "mlp": moe}
         return {"type": "latent_attention", "mixer": dict(latent, kv_from=index - 2), "mlp": moe}
 
-    dubizen = {"architecture": "Dubizen", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+    dubizen = {"architecture": "Dubizen", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
                "layers": [entry(i) for i in range(layers)]}
     others = rekezen_configs(width, layers)
     return {"Dubizen": dubizen, "Rekezen": others["Rekezen"], "Qwen3": others["Qwen3"]}

@@ -367,7 +367,7 @@ static int launch_latent(const void* q, long long q_stride, const void* key_page
 // The (DK, DV) pairs compiled below; 0 for any other.
 extern "C" int fe_latent_attention_supported(int row_dim, int value_dim) {
   return (row_dim == 576 && value_dim == 512) || (row_dim == 320 && value_dim == 256) || (row_dim == 192 && value_dim == 128) ||
-         (row_dim == 128 && value_dim == 96) || (row_dim == 96 && value_dim == 64);
+         (row_dim == 160 && value_dim == 128) || (row_dim == 96 && value_dim == 64);
 }
 
 extern "C" int fe_latent_attention(const void* q, long long q_stride, const void* key_pages, const void* value_pages, void* out,
@@ -387,7 +387,7 @@ extern "C" int fe_latent_attention(const void* q, long long q_stride, const void
   CASE(576, 512);
   CASE(320, 256);
   CASE(192, 128);
-  CASE(128, 96);
+  CASE(160, 128);
   CASE(96, 64);
 #undef CASE
   return FE_BAD_ARGUMENT;

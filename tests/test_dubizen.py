@@ -218,7 +218,7 @@ def test_each_mechanism_alone_through_the_engine(case, tmp_path, monkeypatch):
         "latent_reader": single(du.latent(2, 6, 6, 4, 5, 11, turned=4, base=77.0, source=0), None,
                                 before=du.layer(du.latent(3, 10, 6, 14, 9, 11, turned=4, base=77.0), None)),
         "dense": single(quiet, du.dense(36)),
-        "experts": single(quiet, du.moe(12, 3, 10, shared=6, groups=(4, 2), scale=2.5)),
+        "experts": single(quiet, du.moe(12, 3, 10, shared=6, groups=(4, 2), scale=2.25)),
         "experts_all": single(quiet, du.moe(3, 3, 10, scale=0.5)),
     }[case]
     if case == "no_window":
@@ -326,14 +326,14 @@ def test_expert_choice_reference_against_the_plain_choice():
         router = torch.randn(experts + 1, 12, generator=g)
         correction = torch.randn(experts, generator=g) * 0.3 - 0.2
         chosen, weights, logits = kernel_refs.moe_route_grouped(x, router, correction, experts=experts, top=top, groups=groups,
-                                                                 keep=keep, scale=2.5)
+                                                                 keep=keep, scale=2.25)
         assert logits.shape == (40, experts + 1)
         scores = torch.softmax((x.double() @ router[:experts].double().T), dim=-1)
         for t in range(40):
             want, _ = plain.choose_experts(scores[t], correction.double(), top, groups, keep)
             assert chosen[t].tolist() == want, (experts, t)
             total = sum(float(scores[t, e]) for e in want)
-            assert torch.allclose(weights[t].double(), torch.tensor([float(scores[t, e]) / total * 2.5 for e in want], dtype=F64), atol=1e-5)
+            assert torch.allclose(weights[t].double(), torch.tensor([float(scores[t, e]) / total * 2.25 for e in want], dtype=F64), atol=1e-5)
 
 
 def test_norm_and_activation_references():

@@ -79,11 +79,11 @@ def test_choice_of_experts_within_the_best_groups(tokens, hidden, experts, top, 
     router = (torch.randn(experts + 1, hidden, generator=g) * 0.3).to(dtype)
     correction = torch.randn(experts, generator=g) * 0.2 - 0.1
     chosen, weights, logits = ops.moe_route_grouped(x.to(DEV), router.to(DEV), correction.to(DEV), experts=experts, top=top, groups=groups,
-                                                    keep=keep, scale=2.5)
+                                                    keep=keep, scale=1.75)
     assert logits.shape == (tokens, experts + 1)
     close(logits, x.float() @ router.float().T, dtype, loose=2.0)
     eye = torch.eye(experts + 1)          # the reference on the kernel's logits: x = logits, router = identity
-    want_chosen, want_weights, _ = refs.moe_route_grouped(logits.cpu(), eye, correction, experts=experts, top=top, groups=groups, keep=keep, scale=2.5)
+    want_chosen, want_weights, _ = refs.moe_route_grouped(logits.cpu(), eye, correction, experts=experts, top=top, groups=groups, keep=keep, scale=1.75)
     assert torch.equal(chosen.cpu(), want_chosen)
     close(weights, want_weights, torch.float32, loose=5.0)
 
@@ -121,7 +121,7 @@ def test_weighted_norms_of_q_and_k_heads_before_the_page_write(heads, kv_heads, 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("block_size", [4, 16])
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 24, 16), (6, 3, 64, 64), (8, 2, 128, 128), (2, 2, 10, 6), (3, 1, 96, 32)])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 24, 16), (6, 3, 64, 64), (8, 2, 128, 128), (2, 2, 10, 6), (3, 1, 80, 48)])
 @pytest.mark.parametrize("window", [1, 7, 64, 150])
 def test_one_key_at_the_window_s_edge_with_biases_by_distance(dtype, block_size, heads, kv_heads, dim, vdim, window):
     """Keys whose scores dominate sit just inside and just outside the window of the last token, of the
@@ -192,7 +192,7 @@ def latent_cache(length, row_dim, value_dim, block_size, dtype, g, loud=()):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("block_size", [8, 16, 64])
-@pytest.mark.parametrize("heads,row_dim,value_dim", [(4, 192, 128), (16, 96, 64), (3, 128, 96), (7, 320, 256), (20, 576, 512), (5, 40, 24), (2, 300, 280)])
+@pytest.mark.parametrize("heads,row_dim,value_dim", [(4, 192, 128), (16, 96, 64), (3, 160, 128), (7, 320, 256), (20, 576, 512), (5, 40, 24), (2, 300, 280)])
 def test_attention_over_a_latent_s_rows(dtype, block_size, heads, row_dim, value_dim):
     """One shared cache of rows read by every head: a prompt's portion behind cached rows (its rows span
     several blocks of 64 and end inside one), single tokens at the first position, at page borders and far
