@@ -317,24 +317,49 @@ __global__ __launch_bounds__(256, (DK / 8 + DV / 4 > 160) ? 1 : 2) void latent_a
   }
 }
 
-// out[row] = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), m the largest m_s; the runs in order.
+// out[row] = sum_s o_s 2^(m_s - m) / sum_s l_s 2^(m_s - m), m the largest m_s; the runs in order.  Block per row.
+// The runs are read eight at a time with all loads of a round in flight (a run's index beyond the last reads the
+// last again and is given no weight): one load after the other, each waited for, made the merge as long as
+// the attention itself.
+#define MERGE_ROUND 8
 __global__ __launch_bounds__(128) void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                            bf16_t* __restrict__ out, int splits, int total_rows, int dv) {
   const int row = blockIdx.x;
+  auto stats = [&](int s) { return part_ml + ((size_t)min(s, splits - 1) * total_rows + row) * 2; };
   float top = -INFINITY;
-  for (int s = 0; s < splits; ++s) top = fmaxf(top, part_ml[((size_t)s * total_rows + row) * 2]);
+  for (int s0 = 0; s0 < splits; s0 += MERGE_ROUND) {
+    float m[MERGE_ROUND];
+#pragma unroll
+    for (int j = 0; j < MERGE_ROUND; ++j) m[j] = stats(s0 + j)[0];
+#pragma unroll
+    for (int j = 0; j < MERGE_ROUND; ++j) top = fmaxf(top, m[j]);
+  }
   const float m_use = top > -INFINITY ? top : 0.f;
   float denom = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float* pm = part_ml + ((size_t)s * total_rows + row) * 2;
-    denom += pm[1] * __builtin_amdgcn_exp2f(pm[0] - m_use);
+  for (int s0 = 0; s0 < splits; s0 += MERGE_ROUND) {
+    float m[MERGE_ROUND], l[MERGE_ROUND];
+#pragma unroll
+    for (int j = 0; j < MERGE_ROUND; ++j) {
+      m[j] = stats(s0 + j)[0];
+      l[j] = stats(s0 + j)[1];
+    }
+#pragma unroll
+    for (int j = 0; j < MERGE_ROUND; ++j)
+      if (s0 + j < splits) denom += l[j] * __builtin_amdgcn_exp2f(m[j] - m_use);
   }
   const float inv = denom > 0.f ? 1.f / denom : 0.f;
   for (int d = threadIdx.x; d < dv; d += 128) {
     float acc = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const size_t at = (size_t)s * total_rows + row;
-      acc += part_o[at * dv + d] * __builtin_amdgcn_exp2f(part_ml[at * 2] - m_use);
+    for (int s0 = 0; s0 < splits; s0 += MERGE_ROUND) {
+      float m[MERGE_ROUND], o[MERGE_ROUND];
+#pragma unroll
+      for (int j = 0; j < MERGE_ROUND; ++j) {
+        m[j] = stats(s0 + j)[0];
+        o[j] = part_o[((size_t)min(s0 + j, splits - 1) * total_rows + row) * dv + d];
+      }
+#pragma unroll
+      for (int j = 0; j < MERGE_ROUND; ++j)
+        if (s0 + j < splits) acc += o[j] * __builtin_amdgcn_exp2f(m[j] - m_use);
     }
     out[(size_t)row * dv + d] = float_to_bf16(acc * inv);
   }

@@ -1514,8 +1514,8 @@ def latent_query_pack(q: Tensor, qa: Tensor, inv_freq: Tensor | None, positions:
 
 
 LATENT_TARGET_BLOCKS = 512      # blocks the matrix-core attention over a latent aims at before it stops cutting the keys into runs
-LATENT_MIN_TILES = 4            # ... and the fewest tiles a run may have (8 sequences at 1,024 keys, 16 heads, rows of 576, us a call with the
-                                # merge: 1 run 110, 2 runs 62, 4 runs 40, 8 runs 32, 16 runs 35, 32 runs 51)
+LATENT_MIN_TILES = 2            # ... and the fewest tiles a run may have (8 sequences at 1,024 keys, 16 heads, rows of 576, us a call with the
+                                # merge, in a captured graph: 1 run 110, 2 runs 62, 4 runs 36, 8 runs 24, 16 runs 21, 32 runs 25)
 
 
 def latent_splits(num_seqs: int, max_q_len: int, heads: int, max_ctx: int | None) -> int:
